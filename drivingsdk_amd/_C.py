@@ -1,0 +1,114 @@
+"""Binding layer: the two functions the reference exports from its compiled module
+``mx_driving._C`` (mx_driving/_C/__init__.pyi:67-81, mx_driving/csrc/pybind.cpp:110-111),
+with the checks, output allocation and dtype policy of
+mx_driving/csrc/MultiScaleDeformableAttn.cpp:28-118, over the C ABI of libmxd_msda.so.
+
+Differences from the reference binding, all widening:
+  * bfloat16 is accepted next to float16/float32;
+  * float16/bfloat16 are read natively by the kernels (fp32 accumulation, one rounding at
+    the store) instead of being up-cast to fp32 copies first;
+  * ``num_levels * num_points <= 64`` is not required.
+Work is enqueued on torch's current stream of the tensors' device; nothing synchronises.
+"""
+import torch
+
+from . import _lib
+
+_FLOAT_CODES = {torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_common(value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights):
+    _check(value.dtype in _FLOAT_CODES,
+           f"value: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {value.dtype}")
+    _check(value_spatial_shapes.dtype == torch.int32,
+           f"value_spatial_shapes: int32 tensor expected but got a tensor with dtype: {value_spatial_shapes.dtype}")
+    _check(value_level_start_index.dtype == torch.int32,
+           "value_level_start_index: int32 tensor expected but got a tensor with dtype: "
+           f"{value_level_start_index.dtype}")
+    _check(sampling_locations.dtype in _FLOAT_CODES,
+           "sampling_locations: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: "
+           f"{sampling_locations.dtype}")
+    _check(attention_weights.dtype in _FLOAT_CODES,
+           "attention_weights: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: "
+           f"{attention_weights.dtype}")
+    _check(value.dim() == 4, "value: expected [bs, num_keys, num_heads, embed_dims]")
+    _check(sampling_locations.dim() == 6 and sampling_locations.size(5) == 2,
+           "sampling_locations: expected [bs, num_queries, num_heads, num_levels, num_points, 2]")
+    _check(attention_weights.dim() == 5, "attention_weights: expected [bs, num_queries, num_heads, num_levels, num_points]")
+    _check(value_spatial_shapes.dim() == 2 and value_spatial_shapes.size(1) == 2,
+           "value_spatial_shapes: expected [num_levels, 2]")
+    _check(value.size(3) <= 256, "The number of embedding dimensions should be less than or equal to 256")
+    bs, nk, nh, hd = value.shape
+    nl = value_spatial_shapes.size(0)
+    _, nq, _, nl_attn, npts, _ = sampling_locations.shape
+    _check(sampling_locations.size(0) == bs and sampling_locations.size(2) == nh,
+           "sampling_locations: batch size / num_heads do not match value")
+    _check(tuple(attention_weights.shape) == (bs, nq, nh, nl_attn, npts),
+           "attention_weights: shape does not match sampling_locations")
+    _check(value_level_start_index.numel() == nl, "value_level_start_index: expected [num_levels]")
+    _check(nl_attn >= nl, "sampling_locations carries fewer levels than value_spatial_shapes")
+    tensors = (value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights)
+    _check(all(t.is_cuda for t in tensors),
+           "multi_scale_deformable_attn: all tensors must live on a GPU (this build has no CPU implementation)")
+    _check(all(t.device == value.device for t in tensors), "multi_scale_deformable_attn: tensors are on different devices")
+    return bs, nk, nh, hd, nl, nl_attn, nq, npts
+
+
+def multi_scale_deformable_attn(value, value_spatial_shapes, value_level_start_index, sampling_locations,
+                                attention_weights):
+    """Forward.  Returns output ``[bs, num_queries, num_heads*embed_dims]`` in value's dtype."""
+    dims = _check_common(value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights)
+    bs, nk, nh, hd, nl, nl_attn, nq, npts = dims
+    lib = _lib.load()
+    dt = value.dtype
+    value = value.contiguous()
+    shapes = value_spatial_shapes.contiguous()
+    lsi = value_level_start_index.contiguous()
+    loc = sampling_locations.to(dt).contiguous()
+    attn = attention_weights.to(dt).contiguous()
+    output = torch.empty((bs, nq, nh * hd), dtype=dt, device=value.device)
+    with torch.cuda.device(value.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.mxd_msda_forward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(),
+                                  attn.data_ptr(), output.data_ptr(), _FLOAT_CODES[dt], bs, nk, nh, hd, nl, nl_attn,
+                                  nq, npts, stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return output
+
+
+def multi_scale_deformable_attn_backward(value, shape, level_start_index, location_trans, attn_weight_trans,
+                                         grad_output):
+    """Backward.  Returns (grad_value, grad_sampling_loc, grad_attn_weight) in value's dtype."""
+    dims = _check_common(value, shape, level_start_index, location_trans, attn_weight_trans)
+    bs, nk, nh, hd, nl, nl_attn, nq, npts = dims
+    _check(grad_output.dtype in _FLOAT_CODES,
+           f"grad_output: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {grad_output.dtype}")
+    _check(grad_output.is_cuda and grad_output.device == value.device, "grad_output: must be on value's device")
+    _check(grad_output.numel() == bs * nq * nh * hd, "grad_output: expected [bs, num_queries, num_heads*embed_dims]")
+    lib = _lib.load()
+    dt = value.dtype
+    value = value.contiguous()
+    shapes = shape.contiguous()
+    lsi = level_start_index.contiguous()
+    loc = location_trans.to(dt).contiguous()
+    attn = attn_weight_trans.to(dt).contiguous()
+    gout = grad_output.to(dt).contiguous()
+    grad_value = torch.empty_like(value)
+    grad_loc = torch.empty_like(loc)
+    grad_attn = torch.empty_like(attn)
+    code = _FLOAT_CODES[dt]
+    ws_bytes = lib.mxd_msda_backward_workspace_bytes(code, bs, nk, nh, hd)
+    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=value.device) if ws_bytes else None
+    with torch.cuda.device(value.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.mxd_msda_backward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(), attn.data_ptr(),
+                                   gout.data_ptr(), grad_value.data_ptr(), grad_loc.data_ptr(), grad_attn.data_ptr(),
+                                   workspace.data_ptr() if workspace is not None else None, ws_bytes, code, bs, nk,
+                                   nh, hd, nl, nl_attn, nq, npts, stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return grad_value, grad_loc, grad_attn

@@ -1,0 +1,24 @@
+"""drivingsdk_amd -- multi-scale deformable attention for AMD Instinct MI355X (gfx950).
+
+One operator, behind the reference SDK's own Python API:
+
+    from drivingsdk_amd import multi_scale_deformable_attn
+    out = multi_scale_deformable_attn(value, spatial_shapes, level_start_index,
+                                      sampling_locations, attention_weights)
+
+``import mx_driving`` (the alias package next to this one) exposes the same names under the
+reference's module path.  The compute is hand-written HIP behind a C ABI
+(include/mxd_msda.h -> drivingsdk_amd/lib/libmxd_msda.so); there is no CPU fallback.
+"""
+from . import _C  # noqa: F401
+from .ops.multi_scale_deformable_attn import (  # noqa: F401
+    MultiScaleDeformableAttnFunction,
+    multi_scale_deformable_attn,
+    npu_multi_scale_deformable_attn_function,
+)
+
+__all__ = [
+    "MultiScaleDeformableAttnFunction",
+    "multi_scale_deformable_attn",
+    "npu_multi_scale_deformable_attn_function",
+]

@@ -1,0 +1,298 @@
+// Backward kernel of multi-scale deformable attention for gfx950 (MI355X), wave64.
+//
+// For every sample (b,q,h,l,p) with g = grad_out[b,q,h,:]:
+//   grad_value[row_c] += w_c * attn * g                  (4 corner rows, fp32 atomics)
+//   d_c = dot(value[row_c], g)
+//   grad_attn = sum_c w_c d_c
+//   grad_x = W attn (hh (d2-d1) + lh (d4-d3)),  grad_y = H attn (hw (d3-d1) + lw (d4-d2))
+// Arithmetic: reference kernels/multi_scale_deformable_attn/op_kernel/multi_scale_deformable_attn_grad.cpp:208-249
+// and kernels/multi_scale_deformable_attn/op_kernel/arch35/multi_scale_deformable_attn_grad.cpp:16-145.
+//
+// Structure (same unit/lane layout and LDS staging as the forward kernel):
+//   * geometry per lane -> LDS strip (row offsets, w_c*attn);
+//   * per staged sample the lanes of a unit fetch the 4 corner rows with one buffer load
+//     each, form partial dots with the register-resident grad_out row, and issue the
+//     scatter as buffer atomics whose consecutive lanes hit consecutive floats of a row
+//     (out-of-image corners carry an out-of-range offset: the load yields 0, the atomic is
+//     dropped by the range check);
+//   * partial dots are summed across the unit's lanes with DPP, parked in LDS, and the
+//     geometry lanes turn them into grad_attn / grad_loc and store them coalesced.
+#include "msda_device.h"
+
+namespace mxd {
+
+template <typename T, int VEC, int NPASS>
+__global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
+{
+    constexpr int NE = VEC * NPASS;  // channels per lane
+    constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    i32x4* lvl = reinterpret_cast<i32x4*>(smem);
+    Work wk;
+    if (!decode_block(a.plan, blockIdx.x, a.bs, a.nh, a.nq, &wk)) return;
+
+    for (int i = threadIdx.x; i < a.nl; i += blockDim.x) {
+        i32x4 L;
+        L.x = a.shapes[2 * i];
+        L.y = a.shapes[2 * i + 1];
+        L.z = a.lsi[i];
+        L.w = 0;
+        lvl[i] = L;
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int LPR = a.plan.lanes_per_row;
+    const int lpr_log2 = __builtin_ctz(LPR);
+    const int U = a.plan.units_per_wave;
+    const int g = lane >> lpr_log2;
+    const int c = lane & (LPR - 1);
+
+    // per-wavefront LDS strip: staged samples, then their four reduced dots
+    unsigned char* strip = smem + kMaxLevels * sizeof(i32x4) +
+                           (size_t)wave * U * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4));
+    Entry* stage = reinterpret_cast<Entry*>(strip);
+    f32x4* dots = reinterpret_cast<f32x4*>(strip + (size_t)U * kChunkStride * sizeof(Entry));
+
+    const T* loc = static_cast<const T*>(a.loc);
+    const T* attn = static_cast<const T*>(a.attn);
+    const T* gout = static_cast<const T*>(a.grad_out);
+    T* gloc = static_cast<T*>(a.grad_loc);
+    T* gattn = static_cast<T*>(a.grad_attn);
+
+    const __amdgpu_buffer_rsrc_t vres =
+        make_rsrc(static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes, a.batch_bytes);
+    const __amdgpu_buffer_rsrc_t gres =
+        make_rsrc(reinterpret_cast<const char*>(a.grad_value) + (size_t)wk.b * a.gbatch_bytes, a.gbatch_bytes);
+    const uint32_t head_off = (uint32_t)wk.h * a.hd * sizeof(T);
+    const uint32_t ghead_off = (uint32_t)wk.h * a.hd * 4u;
+
+    uint32_t choff[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        const int ch = (c + p * LPR) * VEC;
+        choff[p] = head_off + (ch < a.hd ? ch * (uint32_t)sizeof(T) : 0u);
+    }
+
+    const int entries = U * kChunk;
+    for (int it = 0; it < a.plan.iters; ++it) {
+        const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
+        if (q0 >= wk.q_end) break;
+
+        // grad_out row of this lane's unit, twice: in the value-load layout (for the dots) and
+        // one float per lane-stride (for the scatter: consecutive lanes -> consecutive floats)
+        const int qg = q0 + g;
+        const bool unit_ok = qg < wk.q_end;
+        const T* grow = gout + (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
+        float gv[NPASS][VEC];
+        float gs[NE];
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            const int ch = (c + p * LPR) * VEC;
+            if (unit_ok && ch < a.hd) {
+                RowIO<T, VEC>::load_global(grow + ch, gv[p]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) gv[p][e] = 0.0f;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const int ch = c + e * LPR;
+            gs[e] = (unit_ok && ch < a.hd) ? to_f32(grow[ch]) : 0.0f;
+        }
+
+        for (int c0 = 0; c0 < a.S; c0 += kChunk) {
+            // ---- geometry -----------------------------------------------------------------
+            for (int i = lane; i < entries; i += kWave) {
+                const int u = i >> 4, sl = i & (kChunk - 1);
+                const int s = c0 + sl, q = q0 + u;
+                const bool active = (q < wk.q_end) && (s < a.S);
+                float x = 0.f, y = 0.f, aw = 0.f;
+                int l = 0;
+                if (active) {
+                    const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;
+                    x = to_f32(loc[2 * e]);
+                    y = to_f32(loc[2 * e + 1]);
+                    aw = to_f32(attn[e]);
+                    l = (int)(((uint32_t)s * a.np_magic) >> 20);
+                }
+                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active);
+                Entry en;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
+                    en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
+                }
+                stage[u * kChunkStride + sl] = en;
+            }
+            wave_lds_sync();
+
+            // ---- gather, dots, scatter ----------------------------------------------------
+            const int ns = (a.S - c0) < kChunk ? (a.S - c0) : kChunk;
+            const Entry* mine = stage + g * kChunkStride;
+            for (int sl = 0; sl < ns; ++sl) {
+                const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
+                const f32x4 w = *reinterpret_cast<const f32x4*>(mine[sl].w);
+                float d[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int p = 0; p < NPASS; ++p) {
+                    typename RowIO<T, VEC>::raw_t raw[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        float v[VEC];
+                        RowIO<T, VEC>::unpack(raw[k], v);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint32_t base = (off[k] << GSHIFT) + ghead_off;
+#pragma unroll
+                    for (int e = 0; e < NE; ++e) {
+                        const int ch = c + e * LPR;
+                        if (ch < a.hd)
+                            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[k] * gs[e], gres, base + ch * 4u, 0, 0);
+                    }
+                }
+                f32x4 dsum;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) dsum[k] = group_sum(d[k], lpr_log2);
+                if (c == 0) dots[g * kChunk + sl] = dsum;
+            }
+            wave_lds_sync();
+
+            // ---- grad_attn / grad_loc from the reduced dots, one sample per lane ----------
+            for (int i = lane; i < entries; i += kWave) {
+                const int u = i >> 4, sl = i & (kChunk - 1);
+                const int s = c0 + sl, q = q0 + u;
+                if ((q < wk.q_end) && (s < a.S)) {
+                    const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;
+                    const float x = to_f32(loc[2 * e]);
+                    const float y = to_f32(loc[2 * e + 1]);
+                    const float aw = to_f32(attn[e]);
+                    const int l = (int)(((uint32_t)s * a.np_magic) >> 20);
+                    const Sample sm = sample_geometry(x, y, lvl[l], a.nk, true);
+                    const f32x4 dd = dots[u * kChunk + sl];
+                    float ga = 0.f, gx = 0.f, gy = 0.f;
+                    if (sm.valid) {
+                        const float hw = 1.0f - sm.lw, hh = 1.0f - sm.lh;
+                        ga = sm.w[0] * dd[0] + sm.w[1] * dd[1] + sm.w[2] * dd[2] + sm.w[3] * dd[3];
+                        gx = sm.Wf * aw * (hh * (dd[1] - dd[0]) + sm.lh * (dd[3] - dd[2]));
+                        gy = sm.Hf * aw * (hw * (dd[2] - dd[0]) + sm.lw * (dd[3] - dd[1]));
+                    }
+                    gattn[e] = from_f32<T>(ga);
+                    gloc[2 * e] = from_f32<T>(gx);
+                    gloc[2 * e + 1] = from_f32<T>(gy);
+                }
+            }
+            wave_lds_sync();
+        }
+
+        // slots of levels that attention_weights carries beyond spatial_shapes: zero gradients
+        const int extra = a.S_full - a.S;
+        if (extra > 0) {
+            for (int i = lane; i < U * extra; i += kWave) {
+                const int u = i / extra, s = a.S + i % extra, q = q0 + u;
+                if (q < wk.q_end) {
+                    const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;
+                    gattn[e] = from_f32<T>(0.f);
+                    gloc[2 * e] = from_f32<T>(0.f);
+                    gloc[2 * e + 1] = from_f32<T>(0.f);
+                }
+            }
+        }
+    }
+}
+
+// ---- helpers on the same stream: zero-fill of the fp32 image, rounding pass ------------------
+__global__ __launch_bounds__(256) void msda_fill_zero_kernel(float* p, size_t n, int head)
+{
+    // [0, head) scalar up to the first 16-byte boundary, then 16-byte stores, then the tail
+    f32x4* body = reinterpret_cast<f32x4*>(p + head);
+    const size_t n4 = (n - head) / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) body[i] = z;
+    if (blockIdx.x == 0) {
+        if ((int)threadIdx.x < head) p[threadIdx.x] = 0.f;
+        const size_t t = head + n4 * 4 + threadIdx.x;
+        if (threadIdx.x < 4 && t < n) p[t] = 0.f;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void msda_round_kernel(const float* src, T* dst, size_t n)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = from_f32<T>(src[i]);
+}
+
+hipError_t launch_fill_zero(float* p, size_t n, hipStream_t stream)
+{
+    if (n == 0) return hipSuccess;
+    size_t head = ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4;
+    if (head > n) head = n;
+    size_t blocks = ((n - head) / 4 + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL(msda_fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, n, (int)head);
+    return hipGetLastError();
+}
+
+hipError_t launch_round(int dtype, const float* src, void* dst, size_t n, hipStream_t stream)
+{
+    if (n == 0) return hipSuccess;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    if (dtype == MXD_DTYPE_F16)
+        hipLaunchKernelGGL(msda_round_kernel<f16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, src,
+                           static_cast<f16_t*>(dst), n);
+    else if (dtype == MXD_DTYPE_BF16)
+        hipLaunchKernelGGL(msda_round_kernel<bf16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, src,
+                           static_cast<bf16_t*>(dst), n);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+template <typename T, int VEC, int NPASS>
+static hipError_t launch_one(const KArgs& a, hipStream_t stream)
+{
+    hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS>), dim3(a.plan.grid), dim3(a.plan.block), a.plan.lds_bytes,
+                       stream, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_dtype(const KArgs& a, hipStream_t stream)
+{
+    const int vec = a.plan.vec, np = a.plan.npass;
+    if (vec == 1 && np == 1) return launch_one<T, 1, 1>(a, stream);
+    if (vec == 1 && np == 2) return launch_one<T, 1, 2>(a, stream);
+    if (vec == 1 && np == 4) return launch_one<T, 1, 4>(a, stream);
+    if (vec == 2 && np == 1) return launch_one<T, 2, 1>(a, stream);
+    if (vec == 2 && np == 2) return launch_one<T, 2, 2>(a, stream);
+    if (vec == 4 && np == 1) return launch_one<T, 4, 1>(a, stream);
+    if constexpr (sizeof(T) == 2) {
+        if (vec == 8 && np == 1) return launch_one<T, 8, 1>(a, stream);
+    }
+    return hipErrorInvalidConfiguration;
+}
+
+hipError_t launch_backward(int dtype, const KArgs& a, hipStream_t stream)
+{
+    switch (dtype) {
+        case MXD_DTYPE_F32: return launch_dtype<float>(a, stream);
+        case MXD_DTYPE_F16: return launch_dtype<f16_t>(a, stream);
+        case MXD_DTYPE_BF16: return launch_dtype<bf16_t>(a, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace mxd

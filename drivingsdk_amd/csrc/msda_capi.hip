@@ -1,0 +1,251 @@
+// C ABI entry points (include/mxd_msda.h): argument checks, launch geometry, enqueue.
+// Host code only; the kernels live in msda_fwd.hip / msda_bwd.hip.
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "msda_device.h"
+
+namespace mxd {
+hipError_t launch_forward(int dtype, const KArgs& a, hipStream_t stream);
+hipError_t launch_backward(int dtype, const KArgs& a, hipStream_t stream);
+hipError_t launch_fill_zero(float* p, size_t n, hipStream_t stream);
+hipError_t launch_round(int dtype, const float* src, void* dst, size_t n, hipStream_t stream);
+}  // namespace mxd
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int elem_size(int dtype)
+{
+    switch (dtype) {
+        case MXD_DTYPE_F32: return 4;
+        case MXD_DTYPE_F16:
+        case MXD_DTYPE_BF16: return 2;
+        default: return 0;
+    }
+}
+
+int env_int(const char* name, int dflt)
+{
+    const char* v = getenv(name);
+    return (v && *v) ? atoi(v) : dflt;
+}
+
+struct Dims {
+    int64_t bs, nk, nh, hd, nl, nl_attn, nq, np;
+};
+
+int check_dims(int dtype, const Dims& d)
+{
+    if (elem_size(dtype) == 0) return fail(MXD_E_DTYPE, "dtype code %d is not float32(0)/float16(1)/bfloat16(2)", dtype);
+    if (d.bs <= 0 || d.nk <= 0 || d.nh <= 0 || d.hd <= 0 || d.nl <= 0 || d.nq <= 0 || d.np <= 0)
+        return fail(MXD_E_SHAPE, "Input Tensor can not be a empty Tensor (bs=%lld nk=%lld nh=%lld hd=%lld nl=%lld nq=%lld np=%lld)",
+                    (long long)d.bs, (long long)d.nk, (long long)d.nh, (long long)d.hd, (long long)d.nl,
+                    (long long)d.nq, (long long)d.np);
+    if (d.hd > 256) return fail(MXD_E_SHAPE, "The number of embedding dimensions should be less than or equal to 256");
+    if (d.nl > mxd::kMaxLevels) return fail(MXD_E_SHAPE, "The number of levels should be less than or equal to %d", mxd::kMaxLevels);
+    if (d.nl_attn < d.nl)
+        return fail(MXD_E_SHAPE, "attention_weights carries %lld levels but spatial_shapes has %lld", (long long)d.nl_attn,
+                    (long long)d.nl);
+    if (d.nl * d.np > 4096 || d.nl * d.np * d.np >= (1 << 20))
+        return fail(MXD_E_SHAPE, "num_levels*num_points = %lld is beyond what this build indexes", (long long)(d.nl * d.np));
+    if (d.nk * d.nh * d.hd * 4 >= (int64_t(1) << 31))
+        return fail(MXD_E_SHAPE, "one batch element of value (num_keys*num_heads*embed_dims = %lld elements) must stay below 2 GiB at 4 bytes per element",
+                    (long long)(d.nk * d.nh * d.hd));
+    if (d.nq >= (int64_t(1) << 31) - 4096 || d.bs >= (1 << 24) || d.nh >= (1 << 16) ||
+        d.nl_attn * d.np >= (int64_t(1) << 24))
+        return fail(MXD_E_SHAPE, "a dimension is beyond what this build indexes");
+    return MXD_OK;
+}
+
+int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_plan* p)
+{
+    const int rc = check_dims(dtype, d);
+    if (rc != MXD_OK) return rc;
+    const int es = elem_size(dtype);
+    if (align_bytes < es) align_bytes = es;
+    int vec = 16 / es;
+    while (vec > 1 && (d.hd % vec != 0 || align_bytes < vec * es)) vec >>= 1;
+    const int lanes_needed = (int)((d.hd + vec - 1) / vec);
+    int lpr = 4;
+    while (lpr < lanes_needed && lpr < mxd::kWave) lpr <<= 1;
+    int npass = (lanes_needed + lpr - 1) / lpr;
+    if (npass == 3) npass = 4;
+    memset(p, 0, sizeof(*p));
+    p->vec = vec;
+    p->lanes_per_row = lpr;
+    p->npass = npass;
+    p->units_per_wave = mxd::kWave / lpr;
+    p->waves_per_block = 4;
+    int iters = env_int(backward ? "MXD_MSDA_BWD_ITERS" : "MXD_MSDA_FWD_ITERS", 1);
+    if (iters < 1) iters = 1;
+    p->iters = iters;
+    p->tile_q = p->units_per_wave * p->waves_per_block * p->iters;
+    const int64_t ntiles = (d.nq + p->tile_q - 1) / p->tile_q;
+    p->ntiles = (int32_t)ntiles;
+    int64_t grid;
+    const int mode_override = env_int("MXD_MSDA_XCD_MODE", -1);
+    if (mode_override != 0 && d.nh % mxd::kNumXcd == 0) {
+        p->xcd_mode = 1;
+        p->heads_per_xcd = (int32_t)(d.nh / mxd::kNumXcd);
+        p->xcds_per_head = 1;
+        p->tiles_per_part = (int32_t)ntiles;
+        grid = (int64_t)mxd::kNumXcd * p->heads_per_xcd * ntiles * d.bs;
+    } else if (mode_override != 0 && mxd::kNumXcd % d.nh == 0) {
+        p->xcd_mode = 2;
+        p->heads_per_xcd = 1;
+        p->xcds_per_head = (int32_t)(mxd::kNumXcd / d.nh);
+        p->tiles_per_part = (int32_t)((ntiles + p->xcds_per_head - 1) / p->xcds_per_head);
+        grid = (int64_t)mxd::kNumXcd * p->tiles_per_part * d.bs;
+    } else {
+        p->xcd_mode = 0;
+        p->heads_per_xcd = 1;
+        p->xcds_per_head = 1;
+        p->tiles_per_part = (int32_t)ntiles;
+        grid = d.bs * d.nh * ntiles;
+    }
+    if (grid >= (int64_t(1) << 31)) return fail(MXD_E_SHAPE, "problem needs %lld workgroups, beyond the launch limit", (long long)grid);
+    p->grid = (uint32_t)grid;
+    p->block = (uint32_t)(p->waves_per_block * mxd::kWave);
+    size_t per_unit = mxd::kChunkStride * sizeof(mxd::Entry);
+    if (backward) per_unit += mxd::kChunk * sizeof(mxd::f32x4);
+    p->lds_bytes = (uint32_t)(mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)p->waves_per_block * p->units_per_wave * per_unit);
+    return MXD_OK;
+}
+
+int ptr_align(const void* p)
+{
+    const uintptr_t v = reinterpret_cast<uintptr_t>(p);
+    int a = 16;
+    while (a > 1 && (v & (uintptr_t)(a - 1))) a >>= 1;
+    return a;
+}
+
+void fill_args(mxd::KArgs* a, int dtype, const Dims& d)
+{
+    const int es = elem_size(dtype);
+    a->bs = (int32_t)d.bs;
+    a->nk = (int32_t)d.nk;
+    a->nh = (int32_t)d.nh;
+    a->hd = (int32_t)d.hd;
+    a->nl = (int32_t)d.nl;
+    a->np = (int32_t)d.np;
+    a->nq = (int32_t)d.nq;
+    a->S = (int32_t)(d.nl * d.np);
+    a->S_full = (int32_t)(d.nl_attn * d.np);
+    a->np_magic = (uint32_t)(((1u << 20) + d.np - 1) / d.np);
+    a->pitch_bytes = (uint32_t)(d.nh * d.hd * es);
+    a->batch_bytes = (uint32_t)(d.nk * d.nh * d.hd * es);
+    a->gbatch_bytes = (uint32_t)(d.nk * d.nh * d.hd * 4);
+}
+
+}  // namespace
+
+extern "C" {
+
+int mxd_msda_version(void) { return MXD_MSDA_VERSION; }
+
+const char* mxd_msda_last_error(void) { return g_err; }
+
+int mxd_msda_make_plan(int backward, int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn,
+                  int64_t nq, int64_t np, int align_bytes, mxd_msda_plan* plan)
+{
+    if (!plan) return fail(MXD_E_NULL, "plan is NULL");
+    const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
+    return make_plan(backward != 0, dtype, d, align_bytes, plan);
+}
+
+int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                     const void* sampling_loc, const void* attn_weight, void* output, int dtype, int64_t bs, int64_t nk,
+                     int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np, void* hip_stream)
+{
+    const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
+    int rc = check_dims(dtype, d);
+    if (rc != MXD_OK) return rc;
+    if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !output)
+        return fail(MXD_E_NULL, "mxd_msda_forward: NULL data pointer");
+    int align = ptr_align(value);
+    if (ptr_align(output) < align) align = ptr_align(output);
+    mxd::KArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = make_plan(0, dtype, d, align, &a.plan);
+    if (rc != MXD_OK) return rc;
+    fill_args(&a, dtype, d);
+    a.value = value;
+    a.shapes = spatial_shapes;
+    a.lsi = level_start_index;
+    a.loc = sampling_loc;
+    a.attn = attn_weight;
+    a.out = output;
+    const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_forward: launch failed: %s", hipGetErrorString(e));
+    return MXD_OK;
+}
+
+size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd)
+{
+    if (elem_size(dtype) != 2 || bs <= 0 || nk <= 0 || nh <= 0 || hd <= 0) return 0;
+    return (size_t)bs * (size_t)nk * (size_t)nh * (size_t)hd * 4;
+}
+
+int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                      const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
+                      void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype, int64_t bs,
+                      int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
+                      void* hip_stream)
+{
+    const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
+    int rc = check_dims(dtype, d);
+    if (rc != MXD_OK) return rc;
+    if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !grad_output || !grad_value ||
+        !grad_loc || !grad_attn)
+        return fail(MXD_E_NULL, "mxd_msda_backward: NULL data pointer");
+    const size_t need = mxd_msda_backward_workspace_bytes(dtype, bs, nk, nh, hd);
+    if (need > 0 && (!workspace || workspace_bytes < need))
+        return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace of %zu bytes required, %zu given", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    float* image = need > 0 ? static_cast<float*>(workspace) : static_cast<float*>(grad_value);
+    if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_msda_backward: grad image is not 4-byte aligned");
+    int align = ptr_align(value);
+    if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
+    mxd::KArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = make_plan(1, dtype, d, align, &a.plan);
+    if (rc != MXD_OK) return rc;
+    fill_args(&a, dtype, d);
+    a.value = value;
+    a.shapes = spatial_shapes;
+    a.lsi = level_start_index;
+    a.loc = sampling_loc;
+    a.attn = attn_weight;
+    a.grad_out = grad_output;
+    a.grad_value = image;
+    a.grad_loc = grad_loc;
+    a.grad_attn = grad_attn;
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    const size_t n = (size_t)bs * nk * nh * hd;
+    hipError_t e = mxd::launch_fill_zero(image, n, stream);
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: zero-fill launch failed: %s", hipGetErrorString(e));
+    e = mxd::launch_backward(dtype, a, stream);
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: launch failed: %s", hipGetErrorString(e));
+    if (need > 0) {
+        e = mxd::launch_round(dtype, image, grad_value, n, stream);
+        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: rounding launch failed: %s", hipGetErrorString(e));
+    }
+    return MXD_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,225 @@
+// Device-side helpers shared by the forward and backward kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "msda_plan.h"
+
+namespace mxd {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+
+typedef _Float16 f16_t;
+typedef __bf16 bf16_t;
+
+// Kernel arguments (passed by value).
+struct KArgs {
+    const void* value;
+    const int32_t* shapes;
+    const int32_t* lsi;
+    const void* loc;
+    const void* attn;
+    void* out;             // forward output
+    const void* grad_out;  // backward only from here
+    float* grad_value;     // fp32 accumulation image of grad_value
+    void* grad_loc;
+    void* grad_attn;
+    int32_t bs, nk, nh, hd, nl, np, nq;
+    int32_t S;             // nl*np: samples per unit that are evaluated
+    int32_t S_full;        // nl_attn*np: samples per unit that are stored
+    uint32_t np_magic;     // ceil(2^20/np): s/np == (s*np_magic)>>20 while s*np < 2^20
+    uint32_t pitch_bytes;  // nh*hd*sizeof(T): distance between neighbouring pixels of value
+    uint32_t batch_bytes;  // nk*pitch_bytes
+    uint32_t gbatch_bytes; // nk*nh*hd*4: one batch element of the fp32 grad image
+    mxd_msda_plan plan;
+};
+
+// One staged sample: byte offsets of its four corner rows inside the batch element's value
+// slice (kInvalidCorner when the corner must not be touched) and their weights.
+struct __align__(16) Entry {
+    uint32_t off[4];
+    float w[4];
+};
+
+// Any offset >= 2^31 is outside every buffer this library binds (slices are < 2 GiB), so the
+// hardware range check turns such loads into zeros and drops such atomics.  0xC0000000
+// stays out of range when shifted left by one (16-bit value offset -> fp32 grad offset) and
+// when a channel offset (< 64 KiB) is added.
+constexpr uint32_t kInvalidCorner = 0xC0000000u;
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
+{
+    // word3 0x00020000: raw buffer, 32-bit data format, no swizzle (gfx9 family encoding)
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// Orders this wavefront's LDS writes before its later LDS reads (and vice versa) without a
+// workgroup barrier: LDS operations of one wavefront complete in order, so it is enough to
+// stop the compiler from moving them across this point.
+__device__ inline void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T>
+__device__ inline float to_f32(T v)
+{
+    return (float)v;
+}
+template <typename T>
+__device__ inline T from_f32(float v)
+{
+    return (T)v;
+}
+
+// ---- row access: VEC elements of T at a byte offset of a bound buffer -> fp32 -------------
+template <typename T, int VEC>
+struct RowIO;
+
+template <typename T, int VEC, int BYTES = VEC * (int)sizeof(T)>
+struct RawBits;
+template <typename T, int VEC>
+struct RawBits<T, VEC, 16> {
+    typedef u32x4 type;
+    static __device__ inline type load(__amdgpu_buffer_rsrc_t r, uint32_t off)
+    {
+        return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+    }
+};
+template <typename T, int VEC>
+struct RawBits<T, VEC, 8> {
+    typedef u32x2 type;
+    static __device__ inline type load(__amdgpu_buffer_rsrc_t r, uint32_t off)
+    {
+        return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+    }
+};
+template <typename T, int VEC>
+struct RawBits<T, VEC, 4> {
+    typedef uint32_t type;
+    static __device__ inline type load(__amdgpu_buffer_rsrc_t r, uint32_t off)
+    {
+        return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+    }
+};
+template <typename T, int VEC>
+struct RawBits<T, VEC, 2> {
+    typedef uint16_t type;
+    static __device__ inline type load(__amdgpu_buffer_rsrc_t r, uint32_t off)
+    {
+        return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0));
+    }
+};
+
+template <typename T, int VEC>
+struct RowIO {
+    typedef T vec_t __attribute__((ext_vector_type(VEC)));
+    typedef typename RawBits<T, VEC>::type raw_t;
+
+    static __device__ inline raw_t load_raw(__amdgpu_buffer_rsrc_t r, uint32_t off)
+    {
+        return RawBits<T, VEC>::load(r, off);
+    }
+    static __device__ inline void unpack(raw_t raw, float (&v)[VEC])
+    {
+        if constexpr (VEC == 1) {
+            v[0] = to_f32(__builtin_bit_cast(T, raw));
+        } else {
+            const vec_t t = __builtin_bit_cast(vec_t, raw);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[i] = to_f32<T>(t[i]);
+        }
+    }
+    // p must be aligned to VEC*sizeof(T)
+    static __device__ inline void load_global(const T* p, float (&v)[VEC])
+    {
+        if constexpr (VEC == 1) {
+            v[0] = to_f32(*p);
+        } else {
+            const vec_t t = *reinterpret_cast<const vec_t*>(p);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) v[i] = to_f32<T>(t[i]);
+        }
+    }
+    static __device__ inline void store_global(T* p, const float (&v)[VEC])
+    {
+        if constexpr (VEC == 1) {
+            *p = from_f32<T>(v[0]);
+        } else {
+            vec_t t;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) t[i] = from_f32<T>(v[i]);
+            *reinterpret_cast<vec_t*>(p) = t;
+        }
+    }
+};
+
+// ---- per-sample geometry ----------------------------------------------------------------
+struct Sample {
+    int32_t pix[4];  // pixel index (within the batch element) of corners (y0,x0) (y0,x1) (y1,x0) (y1,x1)
+    bool cvalid[4];  // corner lies inside the level and inside [0, nk)
+    float w[4];      // bilinear weights, all zero when the sample is invalid
+    float lw, lh;    // fractional parts
+    float Wf, Hf;
+    bool valid;      // sample lies inside (-1, W) x (-1, H) in pixel space; false for NaN/Inf
+};
+
+// level = {H, W, level_start_index, unused}
+__device__ inline Sample sample_geometry(float x, float y, i32x4 level, int32_t nk, bool active)
+{
+    Sample s;
+    const int32_t H = level.x, W = level.y, base = level.z;
+    s.Wf = (float)W;
+    s.Hf = (float)H;
+    const float w_im = __builtin_fmaf(x, s.Wf, -0.5f);
+    const float h_im = __builtin_fmaf(y, s.Hf, -0.5f);
+    s.valid = active && (h_im > -1.0f) && (w_im > -1.0f) && (h_im < s.Hf) && (w_im < s.Wf);
+    const float fx = __builtin_floorf(w_im), fy = __builtin_floorf(h_im);
+    const int32_t x0 = s.valid ? (int32_t)fx : 0;
+    const int32_t y0 = s.valid ? (int32_t)fy : 0;
+    s.lw = w_im - fx;
+    s.lh = h_im - fy;
+    const float hw = 1.0f - s.lw, hh = 1.0f - s.lh;
+    const bool vx0 = x0 >= 0, vx1 = x0 + 1 < W, vy0 = y0 >= 0, vy1 = y0 + 1 < H;
+    const int32_t p00 = base + y0 * W + x0;
+    s.pix[0] = p00;
+    s.pix[1] = p00 + 1;
+    s.pix[2] = p00 + W;
+    s.pix[3] = p00 + W + 1;
+    const bool cv[4] = {vy0 && vx0, vy0 && vx1, vy1 && vx0, vy1 && vx1};
+    const float wt[4] = {hh * hw, hh * s.lw, s.lh * hw, s.lh * s.lw};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        s.cvalid[k] = s.valid && cv[k] && ((uint32_t)s.pix[k] < (uint32_t)nk);
+        s.w[k] = s.valid ? wt[k] : 0.0f;
+    }
+    return s;
+}
+
+// ---- sum over the `lanes` (power of two <= 64) lanes that share a unit; every lane of the
+// group ends with the total.  Uses DPP within 16-lane rows and lane swaps above.
+template <int CTRL>
+__device__ inline float dpp_xchg(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+__device__ inline float group_sum(float v, int lanes_log2)
+{
+    // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror
+    if (lanes_log2 >= 1) v += dpp_xchg<0xB1>(v);
+    if (lanes_log2 >= 2) v += dpp_xchg<0x4E>(v);
+    if (lanes_log2 >= 3) v += dpp_xchg<0x141>(v);
+    if (lanes_log2 >= 4) v += dpp_xchg<0x140>(v);
+    if (lanes_log2 >= 5) v += __shfl_xor(v, 16, 64);
+    if (lanes_log2 >= 6) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+}  // namespace mxd

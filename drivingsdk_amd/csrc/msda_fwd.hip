@@ -1,0 +1,178 @@
+// Forward kernel of multi-scale deformable attention for gfx950 (MI355X), wave64.
+//
+//   out[b,q,h,:] = sum_{l,p} attn[b,q,h,l,p] * bilinear(value_l[b,:,h,:], loc[b,q,h,l,p])
+//
+// Arithmetic: reference kernels/multi_scale_deformable_attn/op_kernel/msda.h:351-539
+// (pixel coordinates, validity, weights) and
+// kernels/multi_scale_deformable_attn/op_kernel/arch35/multi_scale_deformable_attn.cpp:36-80
+// (corner predicates, accumulation).  The structure is this library's own:
+//
+//   * A wavefront works on U = 64/lanes_per_row units (b,q,h) at once; the lanes of a unit
+//     each own `vec` channels, so one corner row is ONE coalesced buffer load (128 B for
+//     head_dim 32 fp32) and the level/point sum stays in fp32 registers -- no reduction
+//     across lanes is ever needed.
+//   * Per pass, every lane first computes the geometry of one or more samples (one sample
+//     per lane, not per unit): validity, floor, the 4 weights times the attention weight,
+//     and the 4 row offsets.  These 32 B per sample go to the wavefront's private LDS strip
+//     and are then read back, broadcast to the lanes of the owning unit.
+//   * Rows are fetched with raw buffer loads bound to the batch element's value slice: a
+//     corner outside the image gets an out-of-range offset and the hardware returns zeros,
+//     so zero padding costs no branch and never touches memory (NaNs in unrelated pixels
+//     cannot leak in).
+#include "msda_device.h"
+
+namespace mxd {
+
+template <typename T, int VEC, int NPASS>
+__global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    i32x4* lvl = reinterpret_cast<i32x4*>(smem);                               // [kMaxLevels]
+    Entry* stage_all = reinterpret_cast<Entry*>(smem + kMaxLevels * sizeof(i32x4));
+
+    Work wk;
+    if (!decode_block(a.plan, blockIdx.x, a.bs, a.nh, a.nq, &wk)) return;      // whole workgroup leaves
+
+    for (int i = threadIdx.x; i < a.nl; i += blockDim.x) {
+        i32x4 L;
+        L.x = a.shapes[2 * i];
+        L.y = a.shapes[2 * i + 1];
+        L.z = a.lsi[i];
+        L.w = 0;
+        lvl[i] = L;
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int lpr_log2 = __builtin_ctz(a.plan.lanes_per_row);
+    const int U = a.plan.units_per_wave;
+    const int g = lane >> lpr_log2;                 // unit slot of this lane
+    const int c = lane & (a.plan.lanes_per_row - 1);  // position inside the row
+    Entry* stage = stage_all + wave * (U * kChunkStride);
+
+    const T* loc = static_cast<const T*>(a.loc);
+    const T* attn = static_cast<const T*>(a.attn);
+    T* out = static_cast<T*>(a.out);
+    const __amdgpu_buffer_rsrc_t vres =
+        make_rsrc(static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes, a.batch_bytes);
+    const uint32_t head_off = (uint32_t)wk.h * a.hd * sizeof(T);
+
+    // channel offsets of this lane for each row pass; lanes past the end of the row read
+    // channel 0 and never store
+    uint32_t choff[NPASS];
+    bool chan_ok[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        const int ch = (c + p * a.plan.lanes_per_row) * VEC;
+        chan_ok[p] = ch < a.hd;
+        choff[p] = head_off + (chan_ok[p] ? ch * (uint32_t)sizeof(T) : 0u);
+    }
+
+    const int entries = U * kChunk;  // staged samples per pass
+    for (int it = 0; it < a.plan.iters; ++it) {
+        const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
+        if (q0 >= wk.q_end) break;  // wavefront-uniform; no workgroup barrier follows
+
+        float acc[NPASS][VEC];
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[p][v] = 0.0f;
+
+        for (int c0 = 0; c0 < a.S; c0 += kChunk) {
+            // ---- geometry: one sample per lane --------------------------------------------
+            for (int i = lane; i < entries; i += kWave) {
+                const int u = i >> 4, sl = i & (kChunk - 1);
+                const int s = c0 + sl, q = q0 + u;
+                const bool active = (q < wk.q_end) && (s < a.S);
+                float x = 0.f, y = 0.f, aw = 0.f;
+                int l = 0;
+                if (active) {
+                    const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;
+                    x = to_f32(loc[2 * e]);
+                    y = to_f32(loc[2 * e + 1]);
+                    aw = to_f32(attn[e]);
+                    l = (int)(((uint32_t)s * a.np_magic) >> 20);
+                }
+                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active);
+                Entry en;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
+                    en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
+                }
+                stage[u * kChunkStride + sl] = en;
+            }
+            wave_lds_sync();
+
+            // ---- gather + weighted sum ----------------------------------------------------
+            const int ns = (a.S - c0) < kChunk ? (a.S - c0) : kChunk;
+            const Entry* mine = stage + g * kChunkStride;
+#pragma unroll 4
+            for (int sl = 0; sl < ns; ++sl) {
+                const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
+                const f32x4 w = *reinterpret_cast<const f32x4*>(mine[sl].w);
+#pragma unroll
+                for (int p = 0; p < NPASS; ++p) {
+                    typename RowIO<T, VEC>::raw_t raw[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        float v[VEC];
+                        RowIO<T, VEC>::unpack(raw[k], v);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) acc[p][e] = __builtin_fmaf(w[k], v[e], acc[p][e]);
+                    }
+                }
+            }
+            wave_lds_sync();
+        }
+
+        const int q = q0 + g;
+        if (q < wk.q_end) {
+            T* orow = out + (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.hd;
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p) {
+                if (chan_ok[p]) RowIO<T, VEC>::store_global(orow + (c + p * a.plan.lanes_per_row) * VEC, acc[p]);
+            }
+        }
+    }
+}
+
+template <typename T, int VEC, int NPASS>
+static hipError_t launch_one(const KArgs& a, hipStream_t stream)
+{
+    hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS>), dim3(a.plan.grid), dim3(a.plan.block), a.plan.lds_bytes,
+                       stream, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_dtype(const KArgs& a, hipStream_t stream)
+{
+    const int vec = a.plan.vec, np = a.plan.npass;
+    if (vec == 1 && np == 1) return launch_one<T, 1, 1>(a, stream);
+    if (vec == 1 && np == 2) return launch_one<T, 1, 2>(a, stream);
+    if (vec == 1 && np == 4) return launch_one<T, 1, 4>(a, stream);
+    if (vec == 2 && np == 1) return launch_one<T, 2, 1>(a, stream);
+    if (vec == 2 && np == 2) return launch_one<T, 2, 2>(a, stream);
+    if (vec == 4 && np == 1) return launch_one<T, 4, 1>(a, stream);
+    if constexpr (sizeof(T) == 2) {
+        if (vec == 8 && np == 1) return launch_one<T, 8, 1>(a, stream);
+    }
+    return hipErrorInvalidConfiguration;
+}
+
+hipError_t launch_forward(int dtype, const KArgs& a, hipStream_t stream)
+{
+    switch (dtype) {
+        case MXD_DTYPE_F32: return launch_dtype<float>(a, stream);
+        case MXD_DTYPE_F16: return launch_dtype<f16_t>(a, stream);
+        case MXD_DTYPE_BF16: return launch_dtype<bf16_t>(a, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace mxd

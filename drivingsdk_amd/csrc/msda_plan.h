@@ -1,0 +1,68 @@
+// Launch geometry and workgroup -> work mapping, shared by host and device code.
+//
+// A "unit" is one (batch, query, head) triple.  `lanes_per_row` lanes of a wavefront share
+// a unit: each moves `vec` channels of a value row per access, so a 64-lane wavefront works
+// on 64/lanes_per_row units side by side.  A workgroup owns `tile_q` consecutive queries of
+// ONE (batch, head) pair.
+//
+// Workgroups are dealt round-robin to the 8 XCDs of an MI355X, each with its own 4 MB L2.
+// The mapping below pins a head to an XCD (or an XCD group), so that an L2 only ever
+// caches the value slice value[:, :, h, :] of its heads -- 1/nh of the tensor -- and walks
+// batch elements one after another.  Correctness does not depend on how the hardware deals
+// workgroups; only the cache hit rate does.
+#pragma once
+#include <stdint.h>
+
+#include "../../include/mxd_msda.h"
+
+#if defined(__HIPCC__)
+#define MXD_HD __host__ __device__
+#else
+#define MXD_HD
+#endif
+
+namespace mxd {
+
+constexpr int kNumXcd = 8;
+constexpr int kWave = 64;
+constexpr int kMaxLevels = 64;
+constexpr int kChunk = 16;           // samples of a unit staged per pass
+constexpr int kChunkStride = 17;     // staged entries per unit incl. one pad entry (LDS banks)
+
+struct Work {
+    int32_t b, h, q_begin, q_end;
+};
+
+// Decode a workgroup index.  Returns false when the workgroup has nothing to do.
+MXD_HD inline bool decode_block(const mxd_msda_plan& p, uint32_t bid, int32_t bs, int32_t nh, int32_t nq, Work* w)
+{
+    int32_t b, h, t;
+    if (p.xcd_mode == 1) {
+        const int32_t x = bid % kNumXcd, j = bid / kNumXcd;
+        const int32_t hs = j % p.heads_per_xcd;
+        const int32_t r = j / p.heads_per_xcd;
+        t = r % p.ntiles;
+        b = r / p.ntiles;
+        h = x * p.heads_per_xcd + hs;
+    } else if (p.xcd_mode == 2) {
+        const int32_t x = bid % kNumXcd, j = bid / kNumXcd;
+        h = x % nh;
+        const int32_t part = x / nh;
+        t = part + p.xcds_per_head * (j % p.tiles_per_part);
+        b = j / p.tiles_per_part;
+    } else {
+        h = bid % nh;
+        const int32_t r = bid / nh;
+        t = r % p.ntiles;
+        b = r / p.ntiles;
+    }
+    if (b >= bs || t >= p.ntiles || h >= nh) return false;
+    w->b = b;
+    w->h = h;
+    w->q_begin = t * p.tile_q;
+    const int32_t e = w->q_begin + p.tile_q;
+    w->q_end = e < nq ? e : nq;
+    return true;
+}
+
+}  // namespace mxd

@@ -1,0 +1,130 @@
+/*
+ * mxd_msda.h -- C ABI of the MI355X (gfx950) multi-scale deformable attention library.
+ *
+ * This is the drop-in boundary for the reference's binding layer: the two functions
+ * the reference exports from its compiled module,
+ *     at::Tensor multi_scale_deformable_attn(value, value_spatial_shapes,
+ *                    value_level_start_index, sampling_locations, attention_weights)
+ *     std::tuple<at::Tensor, at::Tensor, at::Tensor> multi_scale_deformable_attn_backward(
+ *                    ..., grad_output)
+ * (include/csrc/functions.h:58-64, bound in mx_driving/csrc/pybind.cpp:110-111, implemented
+ * in mx_driving/csrc/MultiScaleDeformableAttn.cpp:28-118) reduce, once tensors are
+ * unwrapped, to the entry points below: plain device pointers, sizes, a dtype code and a
+ * HIP stream.  No C++ or torch types cross this boundary.
+ *
+ * Conventions
+ *   - Every data pointer is DEVICE memory, dense row-major, borrowed for the duration of
+ *     the enqueued work; the library allocates and frees nothing.
+ *   - Work is enqueued on `hip_stream` (a hipStream_t; NULL = the default stream) of the
+ *     CURRENT device and the call returns without synchronising.
+ *   - Return value: 0 on success, a negative MXD_E_* code otherwise; the message for the
+ *     calling thread's last failure is returned by mxd_msda_last_error().
+ *   - Thread safe: no mutable global state except the thread-local error message.
+ *
+ * Layouts (T = element type selected by `dtype`)
+ *   value            T   [bs, nk, nh, hd]
+ *   spatial_shapes   i32 [nl, 2]   (H, W) per level
+ *   level_start_idx  i32 [nl]
+ *   sampling_loc     T   [bs, nq, nh, nl_attn, np, 2]   (x, y) normalised to [0, 1]
+ *   attn_weight      T   [bs, nq, nh, nl_attn, np]
+ *   output           T   [bs, nq, nh*hd]
+ *   grad_output      T   [bs, nq, nh*hd]
+ *   grad_value       T   [bs, nk, nh, hd]
+ *   grad_loc         T   like sampling_loc,   grad_attn  T  like attn_weight
+ * nl_attn >= nl: only the first nl levels are sampled; the remaining slots of grad_loc and
+ * grad_attn are written as zero (mx_driving/csrc/MultiScaleDeformableAttn.cpp:97-101).
+ *
+ * Limits (the first two are the reference's, MultiScaleDeformableAttn.cpp:46-48):
+ *   hd <= 256;  nl*np <= 64 is NOT required here (any nl <= 64, any np);
+ *   nk*nh*hd*4 bytes (one batch element of value, counted at 4 bytes per element) < 2 GiB.
+ */
+#ifndef MXD_MSDA_H
+#define MXD_MSDA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MXD_MSDA_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* dtype codes */
+#define MXD_DTYPE_F32 0
+#define MXD_DTYPE_F16 1
+#define MXD_DTYPE_BF16 2
+
+/* error codes */
+#define MXD_OK 0
+#define MXD_E_DTYPE (-1)    /* unsupported dtype code                                   */
+#define MXD_E_SHAPE (-2)    /* a size is non-positive or violates a documented limit    */
+#define MXD_E_NULL (-3)     /* a required pointer is NULL                               */
+#define MXD_E_WORKSPACE (-4) /* workspace missing or too small                          */
+#define MXD_E_LAUNCH (-5)   /* the HIP runtime refused the launch                       */
+
+/* Launch geometry chosen for a problem; filled by mxd_msda_make_plan(), read-only diagnostics.
+ * Replaces the reference's host "tiling" step
+ * (kernels/multi_scale_deformable_attn/op_host/multi_scale_deformable_attn.cpp:32-114,
+ *  kernels/multi_scale_deformable_attn/op_host/multi_scale_deformable_attn_grad.cpp:35-87). */
+typedef struct mxd_msda_plan {
+    int32_t vec;             /* elements of T one lane moves per row access (1,2,4,8)   */
+    int32_t lanes_per_row;   /* power of two, 4..64: lanes that share one value row     */
+    int32_t npass;           /* row passes per lane when hd > lanes_per_row*vec         */
+    int32_t units_per_wave;  /* (query, head) units a wavefront handles side by side    */
+    int32_t waves_per_block;
+    int32_t iters;           /* wave-steps each wavefront runs                          */
+    int32_t tile_q;          /* queries per workgroup = units_per_wave*waves*iters      */
+    int32_t ntiles;          /* query tiles per (batch, head)                           */
+    int32_t xcd_mode;        /* 0 plain; 1 nh % 8 == 0 (heads pinned to an XCD);
+                                2 8 % nh == 0 (several XCDs share a head)               */
+    int32_t heads_per_xcd;   /* mode 1                                                  */
+    int32_t xcds_per_head;   /* mode 2                                                  */
+    int32_t tiles_per_part;  /* mode 2: tiles each of the XCDs sharing a head takes     */
+    uint32_t grid;           /* workgroups                                              */
+    uint32_t block;          /* threads per workgroup                                   */
+    uint32_t lds_bytes;      /* dynamic LDS per workgroup                               */
+} mxd_msda_plan;
+
+/* Library version (MXD_MSDA_VERSION of the build). */
+int mxd_msda_version(void);
+
+/* Message of the calling thread's most recent failed call ("" if none). */
+const char* mxd_msda_last_error(void);
+
+/* Compute the launch geometry for a problem without touching the GPU.
+ * `backward` = 0/1.  `align_bytes` = the largest power of two (<= 16) dividing every data
+ * pointer that will be passed; use 16 when unknown (torch allocations are 256-byte aligned).
+ * Same argument checks and limits as the compute entry points. */
+int mxd_msda_make_plan(int backward, int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
+                       int64_t nl_attn, int64_t nq, int64_t np, int align_bytes, mxd_msda_plan* plan);
+
+/* Forward.  Replaces multi_scale_deformable_attn
+ * (mx_driving/csrc/MultiScaleDeformableAttn.cpp:28-66): reads T natively, accumulates in
+ * fp32, rounds once at the store.  Samples outside the image, and NaN/Inf locations,
+ * contribute nothing. */
+int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                     const void* sampling_loc, const void* attn_weight, void* output, int dtype, int64_t bs,
+                     int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
+                     void* hip_stream);
+
+/* Bytes of scratch mxd_msda_backward needs: 0 for fp32; for fp16/bf16 an fp32 image of
+ * grad_value (bs*nk*nh*hd*4) that the scatter accumulates into before one rounding pass
+ * (the reference keeps the same fp32 buffer, MultiScaleDeformableAttn.cpp:93,103-113). */
+size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd);
+
+/* Backward.  Replaces multi_scale_deformable_attn_backward
+ * (mx_driving/csrc/MultiScaleDeformableAttn.cpp:68-118).  On `hip_stream`, in order:
+ * zero-fills the fp32 accumulation image of grad_value (grad_value itself for fp32, the
+ * workspace otherwise), runs the scatter/reduction kernel, and for fp16/bf16 rounds the
+ * workspace into grad_value.  Every element of the three outputs is written. */
+int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                      const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
+                      void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype,
+                      int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq,
+                      int64_t np, void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXD_MSDA_H */
