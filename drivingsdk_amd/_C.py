@@ -84,10 +84,10 @@ def multi_scale_deformable_attn(value, value_spatial_shapes, value_level_start_i
 def multi_scale_deformable_attn_backward(value, shape, level_start_index, location_trans, attn_weight_trans,
                                          grad_output):
     """Backward.  Returns (grad_value, grad_sampling_loc, grad_attn_weight) in value's dtype."""
-    dims = _check_common(value, shape, level_start_index, location_trans, attn_weight_trans)
-    bs, nk, nh, hd, nl, nl_attn, nq, npts = dims
     _check(grad_output.dtype in _FLOAT_CODES,
            f"grad_output: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {grad_output.dtype}")
+    dims = _check_common(value, shape, level_start_index, location_trans, attn_weight_trans)
+    bs, nk, nh, hd, nl, nl_attn, nq, npts = dims
     _check(grad_output.is_cuda and grad_output.device == value.device, "grad_output: must be on value's device")
     _check(grad_output.numel() == bs * nq * nh * hd, "grad_output: expected [bs, num_queries, num_heads*embed_dims]")
     lib = _lib.load()

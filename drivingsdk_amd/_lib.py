@@ -16,6 +16,7 @@ EXPORTS = (
     "mxd_msda_version",
     "mxd_msda_last_error",
     "mxd_msda_make_plan",
+    "mxd_msda_decode_block",
     "mxd_msda_forward",
     "mxd_msda_backward_workspace_bytes",
     "mxd_msda_backward",
@@ -55,6 +56,9 @@ def load():
     lib.mxd_msda_last_error.argtypes = []
     lib.mxd_msda_make_plan.restype = ci
     lib.mxd_msda_make_plan.argtypes = [ci, ci] + [i64] * 8 + [ci, ctypes.POINTER(Plan)]
+    lib.mxd_msda_decode_block.restype = ci
+    lib.mxd_msda_decode_block.argtypes = [ctypes.POINTER(Plan), ctypes.c_uint32, i64, i64, i64,
+                                          ctypes.POINTER(ctypes.c_int32 * 4)]
     lib.mxd_msda_forward.restype = ci
     lib.mxd_msda_forward.argtypes = [p] * 6 + [ci] + [i64] * 8 + [p]
     lib.mxd_msda_backward_workspace_bytes.restype = ctypes.c_size_t

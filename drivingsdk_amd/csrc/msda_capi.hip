@@ -168,6 +168,19 @@ int mxd_msda_make_plan(int backward, int dtype, int64_t bs, int64_t nk, int64_t 
     return make_plan(backward != 0, dtype, d, align_bytes, plan);
 }
 
+int mxd_msda_decode_block(const mxd_msda_plan* plan, uint32_t block_index, int64_t bs, int64_t nh, int64_t nq,
+                          int32_t work[4])
+{
+    if (!plan || !work) return 0;
+    mxd::Work w;
+    if (!mxd::decode_block(*plan, block_index, (int32_t)bs, (int32_t)nh, (int32_t)nq, &w)) return 0;
+    work[0] = w.b;
+    work[1] = w.h;
+    work[2] = w.q_begin;
+    work[3] = w.q_end;
+    return 1;
+}
+
 int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
                      const void* sampling_loc, const void* attn_weight, void* output, int dtype, int64_t bs, int64_t nk,
                      int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np, void* hip_stream)

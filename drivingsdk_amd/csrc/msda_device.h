@@ -173,20 +173,35 @@ struct Sample {
 // level = {H, W, level_start_index, unused}
 __device__ inline Sample sample_geometry(float x, float y, i32x4 level, int32_t nk, bool active)
 {
+#pragma clang fp contract(off)  // the hi/lo split below must not be re-fused by the compiler
     Sample s;
     const int32_t H = level.x, W = level.y, base = level.z;
     s.Wf = (float)W;
     s.Hf = (float)H;
+    // Correctly rounded pixel coordinates decide validity ...
     const float w_im = __builtin_fmaf(x, s.Wf, -0.5f);
     const float h_im = __builtin_fmaf(y, s.Hf, -0.5f);
     s.valid = active && (h_im > -1.0f) && (w_im > -1.0f) && (h_im < s.Hf) && (w_im < s.Wf);
-    const float fx = __builtin_floorf(w_im), fy = __builtin_floorf(h_im);
+    // ... while cell index and fraction come from the exact product x*W = hi + lo, so that the
+    // fraction carries an absolute error of ~2^-24 instead of half an ulp of the coordinate
+    // (which at W = 150 would already be 4e-6 of a pixel).
+    const float xh = x * s.Wf, xl = __builtin_fmaf(x, s.Wf, -xh);
+    const float yh = y * s.Hf, yl = __builtin_fmaf(y, s.Hf, -yh);
+    const float tx = xh - 0.5f, ty = yh - 0.5f;
+    float fx = __builtin_floorf(tx), fy = __builtin_floorf(ty);
+    s.lw = (tx - fx) + xl;
+    s.lh = (ty - fy) + yl;
+    if (s.lw < 0.0f) { fx -= 1.0f; s.lw += 1.0f; }
+    if (s.lw >= 1.0f) { fx += 1.0f; s.lw -= 1.0f; }
+    if (s.lh < 0.0f) { fy -= 1.0f; s.lh += 1.0f; }
+    if (s.lh >= 1.0f) { fy += 1.0f; s.lh -= 1.0f; }
     const int32_t x0 = s.valid ? (int32_t)fx : 0;
     const int32_t y0 = s.valid ? (int32_t)fy : 0;
-    s.lw = w_im - fx;
-    s.lh = h_im - fy;
     const float hw = 1.0f - s.lw, hh = 1.0f - s.lh;
-    const bool vx0 = x0 >= 0, vx1 = x0 + 1 < W, vy0 = y0 >= 0, vy1 = y0 + 1 < H;
+    // two-sided (unsigned) tests: after the fraction fix-up a cell index may sit one step
+    // outside [-1, size-1] for coordinates within an ulp of a validity edge
+    const bool vx0 = (uint32_t)x0 < (uint32_t)W, vx1 = (uint32_t)(x0 + 1) < (uint32_t)W;
+    const bool vy0 = (uint32_t)y0 < (uint32_t)H, vy1 = (uint32_t)(y0 + 1) < (uint32_t)H;
     const int32_t p00 = base + y0 * W + x0;
     s.pix[0] = p00;
     s.pix[1] = p00 + 1;

@@ -99,6 +99,13 @@ const char* mxd_msda_last_error(void);
 int mxd_msda_make_plan(int backward, int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
                        int64_t nl_attn, int64_t nq, int64_t np, int align_bytes, mxd_msda_plan* plan);
 
+/* Which slice of the problem workgroup `block_index` of a plan works on: writes
+ * {batch, head, first query, one past the last query} to `work` and returns 1, or returns 0
+ * when that workgroup is idle.  Host-side twin of the kernels' own decoding, for checking that
+ * a plan covers every (batch, head, query) exactly once; never needed to run the operator. */
+int mxd_msda_decode_block(const mxd_msda_plan* plan, uint32_t block_index, int64_t bs, int64_t nh, int64_t nq,
+                          int32_t work[4]);
+
 /* Forward.  Replaces multi_scale_deformable_attn
  * (mx_driving/csrc/MultiScaleDeformableAttn.cpp:28-66): reads T natively, accumulates in
  * fp32, rounds once at the store.  Samples outside the image, and NaN/Inf locations,

@@ -1,0 +1,176 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what the header
+declares, argument checking, launch geometry, and the error behaviour of the Python layer."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import drivingsdk_amd
+import mx_driving
+from conftest import ROOT
+from drivingsdk_amd import _C, _lib, workloads
+
+
+def test_library_exports_every_declared_symbol():
+    with open(os.path.join(ROOT, "include", "mxd_msda.h")) as f:
+        header = f.read()
+    declared = set(re.findall(r"\b(mxd_msda_[a-z_]+)\s*\(", header))
+    declared.discard("mxd_msda_plan")
+    assert declared == set(_lib.EXPORTS)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.mxd_msda_version() == 100
+
+
+def test_public_names_match_the_reference_module():
+    for mod in (mx_driving, drivingsdk_amd):
+        assert mod.multi_scale_deformable_attn == mod.MultiScaleDeformableAttnFunction.apply
+        assert callable(mod.npu_multi_scale_deformable_attn_function)
+    assert mx_driving._C.multi_scale_deformable_attn is _C.multi_scale_deformable_attn
+    assert mx_driving._C.multi_scale_deformable_attn_backward is _C.multi_scale_deformable_attn_backward
+
+
+@pytest.mark.parametrize("backward", [0, 1])
+@pytest.mark.parametrize("dims", [
+    # bs, nk, nh, hd, nl, nl_attn, nq, np
+    (2, 19947, 8, 32, 4, 4, 19947, 4),
+    (6, 30825, 8, 32, 4, 4, 9675, 8),
+    (1, 19947, 8, 128, 4, 4, 19947, 4),
+    (1, 2400, 5, 16, 3, 3, 27216, 1),
+    (3, 2400, 4, 37, 5, 5, 301, 3),
+    (1, 2400, 7, 147, 3, 3, 1450, 21),
+    (2, 100, 16, 8, 1, 2, 33, 2),
+    (1, 100, 1, 256, 1, 1, 1, 1),
+    (2, 100, 2, 64, 2, 2, 1000, 4),
+])
+def test_plan_covers_every_unit_exactly_once(backward, dims):
+    bs, nk, nh, hd, nl, nl_attn, nq, npts = dims
+    lib = _lib.load()
+    for dtype in (0, 1, 2):
+        plan = _lib.make_plan(backward, dtype, *dims)
+        assert plan.lanes_per_row * plan.units_per_wave == 64
+        assert plan.vec * plan.lanes_per_row * plan.npass >= hd
+        assert hd % plan.vec == 0
+        assert plan.block == 64 * plan.waves_per_block
+        assert plan.tile_q == plan.units_per_wave * plan.waves_per_block * plan.iters
+        assert plan.lds_bytes <= 64 * 1024
+        seen = {}
+        work = (ctypes.c_int32 * 4)()
+        for bid in range(plan.grid):
+            if not lib.mxd_msda_decode_block(ctypes.byref(plan), bid, bs, nh, nq, ctypes.byref(work)):
+                continue
+            b, h, q0, q1 = work
+            assert 0 <= b < bs and 0 <= h < nh and 0 <= q0 < q1 <= nq and q1 - q0 <= plan.tile_q
+            if plan.xcd_mode == 1:
+                assert h // plan.heads_per_xcd == bid % 8   # a head never leaves its XCD
+            elif plan.xcd_mode == 2:
+                assert h == (bid % 8) % nh
+            assert (b, h, q0) not in seen
+            seen[(b, h, q0)] = q1
+        covered = sum(q1 - q0 for (_, _, q0), q1 in seen.items())
+        assert covered == bs * nh * nq
+        assert len(seen) == bs * nh * plan.ntiles
+
+
+def test_plan_vector_width_follows_alignment_and_head_dim():
+    assert _lib.make_plan(0, 0, 1, 10, 1, 32, 1, 1, 1, 1, 16).vec == 4
+    assert _lib.make_plan(0, 0, 1, 10, 1, 32, 1, 1, 1, 1, 8).vec == 2
+    assert _lib.make_plan(0, 0, 1, 10, 1, 32, 1, 1, 1, 1, 4).vec == 1
+    assert _lib.make_plan(0, 1, 1, 10, 1, 32, 1, 1, 1, 1, 16).vec == 8
+    assert _lib.make_plan(0, 0, 1, 10, 1, 37, 1, 1, 1, 1, 16).vec == 1
+    assert _lib.make_plan(0, 0, 1, 10, 1, 147, 1, 1, 1, 1, 16).npass == 4
+    assert _lib.make_plan(0, 1, 1, 10, 1, 250, 1, 1, 1, 1, 16).vec == 2
+
+
+@pytest.mark.parametrize("dims,fragment", [
+    ((1, 10, 1, 257, 1, 1, 1, 1), "less than or equal to 256"),
+    ((1, 10, 1, 32, 65, 65, 1, 1), "levels"),
+    ((1, 10, 1, 32, 2, 1, 1, 1), "levels"),
+    ((0, 10, 1, 32, 1, 1, 1, 1), "empty"),
+    ((1, 1 << 22, 8, 32, 1, 1, 1, 1), "2 GiB"),
+])
+def test_c_abi_rejects_bad_sizes(dims, fragment):
+    with pytest.raises(RuntimeError) as e:
+        _lib.make_plan(0, 0, *dims)
+    assert fragment in str(e.value)
+    plan = _lib.Plan()
+    assert _lib.load().mxd_msda_make_plan(0, 7, 1, 10, 1, 32, 1, 1, 1, 1, 16, ctypes.byref(plan)) == -1
+    assert _lib.load().mxd_msda_make_plan(0, 0, 1, 10, 1, 32, 1, 1, 1, 1, 16, None) == -3
+
+
+def test_workspace_size():
+    lib = _lib.load()
+    assert lib.mxd_msda_backward_workspace_bytes(0, 2, 100, 8, 32) == 0
+    assert lib.mxd_msda_backward_workspace_bytes(1, 2, 100, 8, 32) == 2 * 100 * 8 * 32 * 4
+    assert lib.mxd_msda_backward_workspace_bytes(2, 2, 100, 8, 32) == 2 * 100 * 8 * 32 * 4
+
+
+def _cpu_inputs(dtype=torch.float32):
+    return workloads.reference_test_inputs([1, 7, 8, 2, 2, 3], dtype=dtype)
+
+
+def test_binding_dtype_checks_raise_before_any_launch():
+    inp = _cpu_inputs()
+    sh, ls = inp.spatial_shapes.int(), inp.level_start_index.int()
+    with pytest.raises(RuntimeError, match="value: float16, bfloat16 or float32"):
+        _C.multi_scale_deformable_attn(inp.value.double(), sh, ls, inp.sampling_locations, inp.attention_weights)
+    with pytest.raises(RuntimeError, match="value_spatial_shapes: int32"):
+        _C.multi_scale_deformable_attn(inp.value, inp.spatial_shapes, ls, inp.sampling_locations,
+                                       inp.attention_weights)
+    with pytest.raises(RuntimeError, match="value_level_start_index: int32"):
+        _C.multi_scale_deformable_attn(inp.value, sh, inp.level_start_index, inp.sampling_locations,
+                                       inp.attention_weights)
+    with pytest.raises(RuntimeError, match="sampling_locations: float16"):
+        _C.multi_scale_deformable_attn(inp.value, sh, ls, inp.sampling_locations.double(), inp.attention_weights)
+    with pytest.raises(RuntimeError, match="attention_weights: float16"):
+        _C.multi_scale_deformable_attn(inp.value, sh, ls, inp.sampling_locations, inp.attention_weights.long())
+    big = torch.zeros(1, 4, 1, 257)
+    with pytest.raises(RuntimeError, match="less than or equal to 256"):
+        _C.multi_scale_deformable_attn(big, sh, ls, inp.sampling_locations, inp.attention_weights)
+    with pytest.raises(RuntimeError, match="grad_output: float16"):
+        _C.multi_scale_deformable_attn_backward(inp.value, sh, ls, inp.sampling_locations, inp.attention_weights,
+                                                inp.grad_output.double())
+
+
+def test_cpu_tensors_are_refused_not_silently_computed():
+    inp = _cpu_inputs()
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        mx_driving.multi_scale_deformable_attn(inp.value, inp.spatial_shapes, inp.level_start_index,
+                                               inp.sampling_locations, inp.attention_weights)
+
+
+def test_empty_tensors_raise_plain_exception_like_the_reference():
+    inp = _cpu_inputs()
+    with pytest.raises(Exception, match="can not be a empty Tensor"):
+        mx_driving.multi_scale_deformable_attn(inp.value[:0], inp.spatial_shapes, inp.level_start_index,
+                                               inp.sampling_locations, inp.attention_weights)
+
+
+def test_deprecated_alias_warns():
+    inp = _cpu_inputs()
+    with pytest.warns(DeprecationWarning):
+        with pytest.raises(RuntimeError):
+            mx_driving.npu_multi_scale_deformable_attn_function(
+                inp.value, inp.spatial_shapes, inp.level_start_index, inp.sampling_locations, inp.attention_weights)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmxd_msda.so"))
+    with pytest.raises(ImportError, match="no CPU or eager fallback"):
+        _lib.load()
+
+
+def test_algorithmic_bytes_match_the_published_table():
+    """Compulsory HBM bytes per call of the five workloads (decimal MB)."""
+    mb = lambda name, dt=torch.float32, bwd=False: workloads.algorithmic_bytes(
+        workloads.make_inputs(name, dtype=dt, scale_queries=1.0), backward=bwd) / 1e6
+    assert abs(mb("tiny") - 4.87) < 0.01
+    assert abs(mb("detr_encoder") - 142.98) < 0.01
+    assert abs(mb("detr_encoder_bwd", bwd=True) - 245.11) < 0.01
+    assert abs(mb("head_dim_128", torch.float16) - 97.02) < 0.01
+    assert abs(mb("bevformer_sca") - 427.16) < 0.01
+    assert abs(mb("bevformer_sca", torch.float16) - 213.58) < 0.01

@@ -1,0 +1,329 @@
+"""Parity of the HIP path (through the public API and the C ABI) with the CPU oracle.
+Everything here needs the GPU; the library is loaded from drivingsdk_amd/lib and the tests
+fail if it is missing."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from drivingsdk_amd import _lib, workloads
+from oracle import msda_oracle as orc
+from util import BWD_FP32, FWD_FP32, HALF, oracle_all, rel_err, run_gpu, to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def _cell_edge_mask(inp):
+    """Samples whose pixel coordinate lies within 2^-20 of an integer on either axis.  The
+    location gradient of bilinear interpolation jumps there (it is the slope of the cell the
+    sample falls in), so a float32 and a float64 evaluation may legitimately pick different
+    sides; such samples are left out of the grad_sampling_locations comparison only."""
+    loc = inp.sampling_locations.double()
+    nl = inp.spatial_shapes.shape[0]
+    hw = inp.spatial_shapes.double()
+    mask = torch.zeros(loc.shape[:-1], dtype=torch.bool)
+    for lvl in range(nl):
+        w_im = loc[:, :, :, lvl, :, 0] * hw[lvl, 1] - 0.5
+        h_im = loc[:, :, :, lvl, :, 1] * hw[lvl, 0] - 0.5
+        dw, dh = (w_im - w_im.round()).abs(), (h_im - h_im.round()).abs()
+        # exactly on an edge is fine: both evaluations are exact there and take the same side
+        near = ((dw > 0) & (dw < 2.0 ** -20)) | ((dh > 0) & (dh < 2.0 ** -20))
+        mask[:, :, :, lvl] = near
+    return mask.numpy()
+
+
+def _check_all(inp, device, fwd_tol, bwd_tol, with_grads=True):
+    ref = oracle_all(inp, with_grads)
+    got = run_gpu(inp, device, with_grads)
+    errs = {}
+    names = ("output", "grad_value", "grad_sampling_locations", "grad_attention_weights")
+    for name, g, r, tol in zip(names, got, ref, (fwd_tol, bwd_tol, bwd_tol, bwd_tol)):
+        if r is None:
+            continue
+        if name == "grad_sampling_locations":
+            edge = _cell_edge_mask(inp)
+            assert edge.mean() < 1e-4, "too many samples sit on a cell edge for this check to mean anything"
+            keep = ~edge[..., None]
+            g, r = g * keep, r * keep
+            errs["cell_edge_samples"] = int(edge.sum())
+        errs[name] = rel_err(g, r)
+        assert errs[name] <= tol, (name, errs)
+    return errs
+
+
+def test_library_is_the_in_tree_build():
+    lib = _lib.load()
+    assert lib.mxd_msda_version() == 100
+    with open("/proc/self/maps") as f:
+        assert any("drivingsdk_amd/lib/libmxd_msda.so" in line for line in f)
+
+
+def test_hand_computed_case_exact(gpu_device, hand_case):
+    c = hand_case
+    inp = workloads.MsdaInputs(c["value"].float(), c["spatial_shapes"], c["level_start_index"],
+                               c["sampling_locations"].float(), c["attention_weights"].float(),
+                               c["grad_output"].float())
+    out, gv, gl, ga = run_gpu(inp, gpu_device)
+    # every quantity of this case is exactly representable; 0.25/0.75 weights are exact too
+    np.testing.assert_allclose(out, c["output"].numpy(), rtol=0, atol=1e-6)
+    np.testing.assert_allclose(gv, c["grad_value"].numpy(), rtol=0, atol=1e-6)
+    np.testing.assert_allclose(gl, c["grad_sampling_locations"].numpy(), rtol=0, atol=1e-5)
+    np.testing.assert_allclose(ga, c["grad_attention_weights"].numpy(), rtol=0, atol=1e-6)
+
+
+def test_tiny_workload_fp32_vs_fixture_and_oracle(gpu_device):
+    from conftest import GOLDEN
+    inp = workloads.make_inputs("tiny", with_grad_output=True)
+    errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+    print("tiny fp32 errors", errs)
+    fx = np.load(os.path.join(GOLDEN, "tiny_expected.npz"))
+    out, gv, gl, ga = run_gpu(inp, gpu_device)
+    assert rel_err(out[0, fx["rows_q"]], fx["output"]) <= FWD_FP32
+    assert rel_err(gv[0, fx["rows_k"]], fx["grad_value"]) <= BWD_FP32
+    assert rel_err(gl[0, fx["rows_q"]], fx["grad_sampling_locations"]) <= BWD_FP32
+    assert rel_err(ga[0, fx["rows_q"]], fx["grad_attention_weights"]) <= BWD_FP32
+
+
+def test_detr_encoder_fp32_full_size(gpu_device):
+    inp = workloads.make_inputs("detr_encoder_bwd")
+    errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+    print("detr_encoder fp32 errors", errs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_bevformer_sca_forward(gpu_device, dtype):
+    inp = workloads.make_inputs("bevformer_sca", dtype=dtype)
+    errs = _check_all(inp, gpu_device, FWD_FP32 if dtype == torch.float32 else HALF, None, with_grads=False)
+    print("bevformer_sca", dtype, errs)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_head_dim_128_forward_and_backward(gpu_device, dtype):
+    inp = workloads.make_inputs("head_dim_128", dtype=dtype, with_grad_output=True)
+    # bfloat16 carries 8 mantissa bits: one rounding of the result is 2^-9 = 1.95e-3 relative
+    tol = HALF if dtype == torch.float16 else 4e-3
+    errs = _check_all(inp, gpu_device, tol, tol)
+    print("head_dim_128", dtype, errs)
+
+
+# shapes of the reference's operator test: [bs, num_queries, embed_dims, num_heads, num_levels, num_points]
+REFERENCE_SHAPES = [
+    [6, 9680, 32, 8, 1, 8],
+    [6, 9680, 32, 8, 4, 4],
+    [6, 9680, 37, 4, 5, 3],
+    [1, 27216, 16, 5, 3, 1],
+    [1, 1450, 64, 6, 1, 2],
+    [1, 1450, 64, 8, 8, 8],
+    [1, 1450, 128, 8, 8, 8],
+    [1, 1450, 256, 8, 8, 8],
+    [1, 1450, 147, 7, 3, 21],
+    [1, 1890, 32, 7, 4, 16],
+]
+
+
+@pytest.mark.parametrize("shape", REFERENCE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_reference_test_shapes_fp32(gpu_device, shape):
+    inp = workloads.reference_test_inputs(shape, seed=sum(shape))
+    errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+    print(shape, errs)
+
+
+def test_reference_fp16_case(gpu_device):
+    inp = workloads.reference_test_inputs([6, 9680, 32, 8, 4, 4], dtype=torch.float16, seed=7)
+    errs = _check_all(inp, gpu_device, HALF, HALF)
+    print("fp16", errs)
+
+
+@pytest.mark.parametrize("fill", [float("nan"), float("inf")])
+def test_nan_and_inf_inputs_give_exact_zeros(gpu_device, fill):
+    inp = workloads.reference_test_inputs([6, 9680, 32, 8, 4, 4], fill=fill)
+    for arr in run_gpu(inp, gpu_device):
+        assert np.all(arr == 0.0)
+
+
+def test_zero_padding_is_exact(gpu_device):
+    """Samples at and beyond the validity edges: same zero / non-zero pattern as the oracle,
+    exact zeros outside, and NaNs in pixels a sample does not touch never leak."""
+    # power-of-two sizes: every pixel coordinate below is exact in float32 and float64 alike,
+    # so the GPU and the oracle must agree on which corners exist, not only on the numbers
+    H, W = 4, 8
+    shapes, lsi = workloads.level_tensors(((H, W),))
+    xs = [(w + 0.5) / W for w in (-1.5, -1.0, -0.75, -0.5, 0.0, 0.5, W - 1.5, W - 1.0, W - 0.75, W - 0.5, W, W + 0.5)]
+    ys = [(h + 0.5) / H for h in (-1.5, -1.0, -0.75, -0.5, 0.0, 0.5, H - 1.5, H - 1.0, H - 0.75, H - 0.5, H, H + 0.5)]
+    pts = torch.tensor([(x, y) for x in xs for y in ys], dtype=torch.float32)
+    nq = pts.shape[0]
+    g = torch.Generator().manual_seed(5)
+    value = torch.randn(1, H * W, 2, 8, generator=g)
+    loc = pts.view(1, nq, 1, 1, 1, 2).expand(1, nq, 2, 1, 1, 2).contiguous()
+    attn = torch.ones(1, nq, 2, 1, 1)
+    gout = torch.randn(1, nq, 16, generator=g)
+    inp = workloads.MsdaInputs(value, shapes, lsi, loc, attn, gout)
+    ref = oracle_all(inp)
+    got = run_gpu(inp, gpu_device)
+    for g_, r_ in zip(got, ref):
+        assert np.array_equal(g_ == 0.0, r_ == 0.0)
+    assert rel_err(got[0], ref[0]) <= FWD_FP32
+    # a NaN pixel poisons only the samples whose in-image corners include it
+    value2 = value.clone()
+    value2[0, 0] = float("nan")  # pixel (0,0)
+    inp2 = inp._replace(value=value2)
+    out2 = run_gpu(inp2, gpu_device, with_grads=False)[0]
+    w_im = pts[:, 0].double() * W - 0.5
+    h_im = pts[:, 1].double() * H - 0.5
+    touches = ((w_im > -1) & (w_im < 1) & (h_im > -1) & (h_im < 1)).numpy()
+    assert np.array_equal(np.isnan(out2[0]).any(-1), touches)
+
+
+def test_more_attention_levels_than_spatial_shapes(gpu_device):
+    """Extra level slots are ignored in the forward pass and receive zero gradients."""
+    g = torch.Generator().manual_seed(11)
+    shapes, lsi = workloads.level_tensors(((9, 7), (4, 6)))
+    nk = int(shapes.prod(1).sum())
+    value = torch.randn(2, nk, 4, 16, generator=g)
+    loc = torch.rand(2, 50, 4, 3, 2, 2, generator=g)
+    attn = torch.rand(2, 50, 4, 3, 2, generator=g)
+    gout = torch.randn(2, 50, 64, generator=g)
+    inp = workloads.MsdaInputs(value, shapes, lsi, loc, attn, gout)
+    errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+    got = run_gpu(inp, gpu_device)
+    assert np.all(got[2][:, :, :, 2:] == 0) and np.all(got[3][:, :, :, 2:] == 0)
+    print(errs)
+
+
+@pytest.mark.parametrize("hd,nh,dtype", [(1, 3, torch.float32), (2, 8, torch.float16), (6, 2, torch.float32),
+                                         (12, 16, torch.float32), (20, 1, torch.bfloat16), (250, 2, torch.float32),
+                                         (255, 1, torch.float16), (24, 8, torch.float16), (200, 4, torch.bfloat16)])
+def test_odd_head_dims_and_head_counts(gpu_device, hd, nh, dtype):
+    g = torch.Generator().manual_seed(hd * 100 + nh)
+    levels = ((11, 13), (5, 7), (1, 1))
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    nq, npts, bs = 77, 5, 2
+    value = torch.randn(bs, nk, nh, hd, generator=g)
+    loc = torch.rand(bs, nq, nh, 3, npts, 2, generator=g) * 1.2 - 0.1
+    attn = torch.rand(bs, nq, nh, 3, npts, generator=g)
+    gout = torch.randn(bs, nq, nh * hd, generator=g)
+    inp = workloads.MsdaInputs(*[t.to(dtype) if t.is_floating_point() else t for t in
+                                 (value, shapes, lsi, loc, attn, gout)])
+    tol_f, tol_b = (FWD_FP32, BWD_FP32) if dtype == torch.float32 else \
+        ((HALF, HALF) if dtype == torch.float16 else (4e-3, 4e-3))
+    errs = _check_all(inp, gpu_device, tol_f, tol_b)
+    print(hd, nh, dtype, errs)
+
+
+def test_unaligned_and_non_contiguous_inputs(gpu_device):
+    """Views with an odd storage offset and strided layouts go through the same path."""
+    import mx_driving
+    inp = workloads.reference_test_inputs([2, 300, 32, 8, 2, 4], seed=3)
+    ref = oracle_all(inp, with_grads=False)[0]
+    d = to_device(inp, gpu_device)
+    # value at a 4-byte (not 16-byte) aligned address
+    buf = torch.empty(d.value.numel() + 1, device=gpu_device)
+    v_off = buf[1:].view_as(d.value)
+    v_off.copy_(d.value)
+    assert v_off.data_ptr() % 16 == 4
+    out = mx_driving.multi_scale_deformable_attn(v_off, d.spatial_shapes, d.level_start_index,
+                                                 d.sampling_locations, d.attention_weights)
+    assert rel_err(out.double().cpu().numpy(), ref) <= FWD_FP32
+    # non-contiguous value (transposed storage) and locations
+    v_nc = d.value.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    l_nc = d.sampling_locations.flip(-1).contiguous().flip(-1)
+    assert not v_nc.is_contiguous()
+    out = mx_driving.multi_scale_deformable_attn(v_nc, d.spatial_shapes, d.level_start_index, l_nc,
+                                                 d.attention_weights)
+    assert rel_err(out.double().cpu().numpy(), ref) <= FWD_FP32
+
+
+def test_int64_metadata_and_mixed_float_dtypes_are_coerced(gpu_device):
+    import mx_driving
+    inp = workloads.reference_test_inputs([1, 200, 32, 8, 2, 4], seed=4)
+    ref = oracle_all(inp, with_grads=False)[0]
+    d = to_device(inp, gpu_device)
+    assert d.spatial_shapes.dtype == torch.int64
+    out = mx_driving.multi_scale_deformable_attn(d.value, d.spatial_shapes, d.level_start_index,
+                                                 d.sampling_locations.double(), d.attention_weights.half())
+    assert out.dtype == torch.float32
+    # attention weights went through float16 here: compare loosely
+    assert rel_err(out.double().cpu().numpy(), ref) <= HALF
+
+
+def test_autocast_runs_in_float32(gpu_device):
+    import mx_driving
+    inp = workloads.reference_test_inputs([1, 200, 32, 8, 2, 4], seed=5)
+    ref = oracle_all(inp, with_grads=False)[0]
+    d = to_device(inp, gpu_device)
+    with torch.autocast("cuda", dtype=torch.float16):
+        out = mx_driving.multi_scale_deformable_attn(d.value.half(), d.spatial_shapes, d.level_start_index,
+                                                     d.sampling_locations, d.attention_weights)
+    assert out.dtype == torch.float32
+    assert rel_err(out.double().cpu().numpy(), ref) <= HALF
+
+
+def test_runs_on_a_side_stream_and_is_repeatable(gpu_device):
+    import mx_driving
+    inp = workloads.make_inputs("tiny", with_grad_output=True)
+    d = to_device(inp, gpu_device)
+    ref = oracle_all(inp)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        outs = []
+        for _ in range(3):
+            v = d.value.clone().requires_grad_()
+            out = mx_driving.multi_scale_deformable_attn(v, d.spatial_shapes, d.level_start_index,
+                                                         d.sampling_locations, d.attention_weights)
+            out.backward(d.grad_output)
+            outs.append((out.detach(), v.grad))
+    s.synchronize()
+    for out, gv in outs:
+        assert torch.equal(out, outs[0][0])                       # forward is deterministic
+        assert rel_err(gv.double().cpu().numpy(), ref[1]) <= BWD_FP32  # atomics: order-dependent rounding only
+
+
+def test_linearity_at_full_size(gpu_device):
+    """Size-independent property at the benchmark shape: linear in value and in the weights."""
+    import mx_driving
+    d = to_device(workloads.make_inputs("detr_encoder"), gpu_device)
+    f = lambda v, a: mx_driving.multi_scale_deformable_attn(v, d.spatial_shapes, d.level_start_index,
+                                                            d.sampling_locations, a)
+    base = f(d.value, d.attention_weights)
+    assert torch.equal(f(2 * d.value, d.attention_weights), 2 * base)       # scaling by 2 is exact
+    assert torch.equal(f(d.value, 0.5 * d.attention_weights), 0.5 * base)
+    other = torch.randn_like(d.value)
+    lhs = f(d.value + other, d.attention_weights)
+    rhs = base + f(other, d.attention_weights)
+    assert rel_err(lhs.double().cpu().numpy(), rhs.double().cpu().numpy()) <= FWD_FP32
+
+
+def test_c_abi_direct_call_and_error_codes(gpu_device):
+    """Straight through the C ABI with raw pointers (what a non-Python host would do)."""
+    lib = _lib.load()
+    inp = workloads.make_inputs("tiny")
+    d = to_device(inp, gpu_device)
+    shapes, lsi = d.spatial_shapes.int(), d.level_start_index.int()
+    bs, nk, nh, hd = d.value.shape
+    _, nq, _, nl, npts, _ = d.sampling_locations.shape
+    out = torch.empty(bs, nq, nh * hd, device=gpu_device)
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = lib.mxd_msda_forward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), d.sampling_locations.data_ptr(),
+                              d.attention_weights.data_ptr(), out.data_ptr(), 0, bs, nk, nh, hd, nl, nl, nq, npts,
+                              stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = oracle_all(inp, with_grads=False)[0]
+    assert rel_err(out.double().cpu().numpy(), ref) <= FWD_FP32
+    # error paths never launch
+    assert lib.mxd_msda_forward(None, shapes.data_ptr(), lsi.data_ptr(), d.sampling_locations.data_ptr(),
+                                d.attention_weights.data_ptr(), out.data_ptr(), 0, bs, nk, nh, hd, nl, nl, nq, npts,
+                                stream) == -3
+    assert lib.mxd_msda_forward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(),
+                                d.sampling_locations.data_ptr(), d.attention_weights.data_ptr(), out.data_ptr(), 0,
+                                bs, nk, nh, 257, nl, nl, nq, npts, stream) == -2
+    assert "256" in _lib.last_error()
+    # fp16 backward without a workspace is refused
+    assert lib.mxd_msda_backward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(),
+                                 d.sampling_locations.data_ptr(), d.attention_weights.data_ptr(), out.data_ptr(),
+                                 out.data_ptr(), out.data_ptr(), out.data_ptr(), None, 0, 1, bs, nk, nh, hd, nl, nl,
+                                 nq, npts, stream) == -4
