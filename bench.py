@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the multi-scale deformable attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+A step is one forward + backward of the operator through the public API on one batch of
+seeded synthetic input that is already resident in HBM.  The default workload is the
+Deformable-DETR encoder shape (bs 2, 19947 queries = keys, 8 heads x 32, 4 levels, 4 points,
+float32).  Prints ONE JSON line: whole-step throughput in queries/s, the HBM roofline of the
+dominant kernel (timed live with HIP events on the launch stream), per-kernel figures, and
+the CPU oracle timed on the host cores of the same box as a reported baseline.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+
+def _event_ms(fn, iters, warmup):
+    """Average duration of fn() in ms from a HIP event pair on the current stream."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def _kernel_times(d, iters, warmup):
+    """Raw C-ABI launches of the three kernels of a step, each timed alone."""
+    import torch
+
+    from drivingsdk_amd import _lib
+
+    lib = _lib.load()
+    dt = d.value.dtype
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dt]
+    shapes, lsi = d.spatial_shapes.int().contiguous(), d.level_start_index.int().contiguous()
+    bs, nk, nh, hd = d.value.shape
+    _, nq, _, nl, npts, _ = d.sampling_locations.shape
+    out = torch.empty(bs, nq, nh * hd, dtype=dt, device=d.value.device)
+    gv, gl, ga = torch.zeros_like(d.value), torch.empty_like(d.sampling_locations), torch.empty_like(d.attention_weights)
+    ws_bytes = lib.mxd_msda_backward_workspace_bytes(code, bs, nk, nh, hd)
+    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=d.value.device)
+    stream = torch.cuda.current_stream().cuda_stream
+    dims = (bs, nk, nh, hd, nl, nl, nq, npts)
+
+    def fwd():
+        rc = lib.mxd_msda_forward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(),
+                                  d.sampling_locations.data_ptr(), d.attention_weights.data_ptr(), out.data_ptr(),
+                                  code, *dims, stream)
+        assert rc == 0, _lib.last_error()
+
+    def bwd(flags):
+        rc = lib.mxd_msda_backward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(),
+                                   d.sampling_locations.data_ptr(), d.attention_weights.data_ptr(),
+                                   d.grad_output.data_ptr(), gv.data_ptr(), gl.data_ptr(), ga.data_ptr(),
+                                   ws.data_ptr() if ws_bytes else None, ws_bytes, code, *dims, flags, stream)
+        assert rc == 0, _lib.last_error()
+
+    res = {"forward_ms": _event_ms(fwd, iters, warmup), "backward_with_zero_fill_ms": _event_ms(lambda: bwd(0), iters, warmup)}
+    if code == 0:
+        # scatter kernel alone: accumulate into the (already initialised) gradient image
+        res["backward_kernel_ms"] = _event_ms(lambda: bwd(_lib.BWD_ACCUMULATE), iters, warmup)
+    else:
+        res["backward_kernel_ms"] = None
+    return res
+
+
+def _cpu_baseline(inp, max_seconds=25.0):
+    """The CPU oracle (grid_sample formulation, float32, autograd backward) on the host cores:
+    whole forward+backward iterations of the same workload, as many as fit the time bound."""
+    import torch
+
+    from oracle import msda_oracle as orc
+
+    threads = torch.get_num_threads()
+    times = []
+    t_begin = time.perf_counter()
+    it = 0
+    while True:
+        t0 = time.perf_counter()
+        orc.msda_grid_sample_fwd_bwd(inp.value, inp.spatial_shapes, inp.sampling_locations, inp.attention_weights,
+                                     inp.grad_output, dtype=torch.float32)
+        t1 = time.perf_counter()
+        if it > 0:  # first iteration is a warm-up
+            times.append(t1 - t0)
+        it += 1
+        if len(times) >= 5 or (time.perf_counter() - t_begin) > max_seconds and times:
+            break
+    med = statistics.median(times)
+    nqueries = inp.sampling_locations.shape[0] * inp.sampling_locations.shape[1]
+    return {"value": nqueries / med, "unit": "queries/s", "cores": threads, "kind": "port",
+            "ms_per_step": med * 1e3,
+            "sample": f"{len(times)} timed forward+backward iterations (median) of the full workload after 1 warm-up, "
+                      f"torch grid_sample formulation in float32 with {threads} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="detr_encoder_bwd")
+    ap.add_argument("--dtype", default="float32", choices=["float32", "float16", "bfloat16"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this operator runs on one GPU; --gpus must be 1 (no multi-GPU path exists in this build)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import mx_driving
+    from drivingsdk_amd import _lib, workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _lib.load()
+    dev = torch.device("cuda", 0)
+    dtype = getattr(torch, args.dtype)
+    inp = workloads.make_inputs(args.workload, dtype=dtype, with_grad_output=True)
+    d = workloads.MsdaInputs(*[t.to(dev) for t in inp])
+    value = d.value.clone().requires_grad_()
+    loc = d.sampling_locations.clone().requires_grad_()
+    attn = d.attention_weights.clone().requires_grad_()
+
+    def step():
+        value.grad = loc.grad = attn.grad = None
+        out = mx_driving.multi_scale_deformable_attn(value, d.spatial_shapes, d.level_start_index, loc, attn)
+        out.backward(d.grad_output)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    bs, nq = loc.shape[0], loc.shape[1]
+    queries = bs * nq
+    bytes_fwd = workloads.algorithmic_bytes(inp, backward=False)
+    bytes_bwd = workloads.algorithmic_bytes(inp, backward=True)
+
+    k = _kernel_times(d, iters=max(args.steps, 50), warmup=max(args.warmup, 10))
+
+    def roof(nbytes, ms, kernel):
+        achieved = nbytes / (ms * 1e-3) / 1e9
+        return {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": nbytes, "kernel_ms": ms}
+
+    roof_fwd = roof(bytes_fwd, k["forward_ms"], "msda_fwd_kernel")
+    bwd_ms = k["backward_kernel_ms"] if k["backward_kernel_ms"] is not None else k["backward_with_zero_fill_ms"]
+    roof_bwd = roof(bytes_bwd, bwd_ms, "msda_bwd_kernel")
+    dominant = roof_bwd if bwd_ms >= k["forward_ms"] else roof_fwd
+
+    cfg = workloads.WORKLOADS[args.workload]
+    result = {
+        "metric": "MSDA fwd+bwd queries/s & achieved HBM GB/s (% roofline), Deformable-DETR enc shape",
+        "value": queries * args.steps / elapsed,
+        "unit": "queries/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"float32": "f32", "float16": "f16", "bfloat16": "bf16"}[args.dtype],
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: forward+backward, bs={bs}, queries={nq}, keys={inp.value.shape[1]}, "
+                               f"heads={cfg['nh']}x{cfg['hd']}, levels={len(cfg['levels'])}, points={cfg['np']}",
+                   "levels": [list(l) for l in cfg["levels"]], "step": "forward+backward through the autograd Function"},
+        "roofline": dominant,
+        "roofline_forward": roof_fwd,
+        "roofline_backward": roof_bwd,
+        "kernels": {**k, "forward_queries_per_s": queries / (k["forward_ms"] * 1e-3),
+                    "fwd_plus_bwd_kernels_ms": k["forward_ms"] + k["backward_with_zero_fill_ms"],
+                    "fwd_plus_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) /
+                    ((k["forward_ms"] + k["backward_with_zero_fill_ms"]) * 1e-3) / 1e9},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = _cpu_baseline(inp)
+        result["speedup_vs_cpu_baseline"] = result["value"] / result["cpu_baseline"]["value"]
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -109,6 +109,6 @@ def multi_scale_deformable_attn_backward(value, shape, level_start_index, locati
         rc = lib.mxd_msda_backward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(), attn.data_ptr(),
                                    gout.data_ptr(), grad_value.data_ptr(), grad_loc.data_ptr(), grad_attn.data_ptr(),
                                    workspace.data_ptr() if workspace is not None else None, ws_bytes, code, bs, nk,
-                                   nh, hd, nl, nl_attn, nq, npts, stream)
+                                   nh, hd, nl, nl_attn, nq, npts, 0, stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return grad_value, grad_loc, grad_attn

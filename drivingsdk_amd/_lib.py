@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libmxd_msda.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
+BWD_ACCUMULATE = 1
 
 EXPORTS = (
     "mxd_msda_version",
@@ -64,7 +65,7 @@ def load():
     lib.mxd_msda_backward_workspace_bytes.restype = ctypes.c_size_t
     lib.mxd_msda_backward_workspace_bytes.argtypes = [ci] + [i64] * 4
     lib.mxd_msda_backward.restype = ci
-    lib.mxd_msda_backward.argtypes = [p] * 10 + [ctypes.c_size_t, ci] + [i64] * 8 + [p]
+    lib.mxd_msda_backward.argtypes = [p] * 10 + [ctypes.c_size_t, ci] + [i64] * 8 + [ci, p]
     _lib = lib
     return lib
 

@@ -218,7 +218,7 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
                       const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
                       void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype, int64_t bs,
                       int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
-                      void* hip_stream)
+                      int flags, void* hip_stream)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     int rc = check_dims(dtype, d);
@@ -230,6 +230,8 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace of %zu bytes required, %zu given", need,
                     workspace ? workspace_bytes : (size_t)0);
+    if ((flags & MXD_BWD_ACCUMULATE) && need > 0)
+        return fail(MXD_E_DTYPE, "mxd_msda_backward: MXD_BWD_ACCUMULATE is only available for float32");
     float* image = need > 0 ? static_cast<float*>(workspace) : static_cast<float*>(grad_value);
     if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_msda_backward: grad image is not 4-byte aligned");
     int align = ptr_align(value);
@@ -250,7 +252,8 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     a.grad_attn = grad_attn;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * nk * nh * hd;
-    hipError_t e = mxd::launch_fill_zero(image, n, stream);
+    hipError_t e = hipSuccess;
+    if (!(flags & MXD_BWD_ACCUMULATE)) e = mxd::launch_fill_zero(image, n, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: zero-fill launch failed: %s", hipGetErrorString(e));
     e = mxd::launch_backward(dtype, a, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: launch failed: %s", hipGetErrorString(e));

@@ -326,4 +326,4 @@ def test_c_abi_direct_call_and_error_codes(gpu_device):
     assert lib.mxd_msda_backward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(),
                                  d.sampling_locations.data_ptr(), d.attention_weights.data_ptr(), out.data_ptr(),
                                  out.data_ptr(), out.data_ptr(), out.data_ptr(), None, 0, 1, bs, nk, nh, hd, nl, nl,
-                                 nq, npts, stream) == -4
+                                 nq, npts, 0, stream) == -4
