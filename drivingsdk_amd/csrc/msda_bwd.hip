@@ -11,12 +11,13 @@
 // Structure (same unit/lane layout and LDS staging as the forward kernel):
 //   * geometry per lane -> LDS strip (row offsets, w_c*attn);
 //   * per staged sample the lanes of a unit fetch the 4 corner rows with one buffer load
-//     each, form partial dots with the register-resident grad_out row, and issue the
-//     scatter as buffer atomics whose consecutive lanes hit consecutive floats of a row
-//     (out-of-image corners carry an out-of-range offset: the load yields 0, the atomic is
-//     dropped by the range check);
-//   * partial dots are summed across the unit's lanes with DPP, parked in LDS, and the
-//     geometry lanes turn them into grad_attn / grad_loc and store them coalesced.
+//     each and form partial dots with the register-resident grad_out row; the partial dots
+//     are summed across the unit's lanes with DPP and parked in LDS;
+//   * the scatter then walks the staged samples again with a row-contiguous lane layout and
+//     issues buffer atomics (out-of-image corners carry an out-of-range offset: the load
+//     yields 0, the atomic is dropped by the hardware range check);
+//   * the geometry lanes turn the reduced dots into grad_attn / grad_loc and store them
+//     coalesced.
 #include "msda_device.h"
 
 namespace mxd {
@@ -24,7 +25,6 @@ namespace mxd {
 template <typename T, int VEC, int NPASS>
 __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
-    constexpr int NE = VEC * NPASS;  // channels per lane
     constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
 
     extern __shared__ __align__(16) unsigned char smem[];
@@ -49,6 +49,9 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     const int U = a.plan.units_per_wave;
     const int g = lane >> lpr_log2;
     const int c = lane & (LPR - 1);
+    // lanes per row in the scatter phase: the power of two covering head_dim, within [LPR, 64]
+    int span_log2 = lpr_log2;
+    while ((1 << span_log2) < a.hd && span_log2 < 6) ++span_log2;
 
     // per-wavefront LDS strip: staged samples, then their four reduced dots
     unsigned char* strip = smem + kMaxLevels * sizeof(i32x4) +
@@ -81,13 +84,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
         if (q0 >= wk.q_end) break;
 
-        // grad_out row of this lane's unit, twice: in the value-load layout (for the dots) and
-        // one float per lane-stride (for the scatter: consecutive lanes -> consecutive floats)
+        // grad_out row of this lane's unit in the value-load layout (for the dots)
         const int qg = q0 + g;
         const bool unit_ok = qg < wk.q_end;
         const T* grow = gout + (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
         float gv[NPASS][VEC];
-        float gs[NE];
 #pragma unroll
         for (int p = 0; p < NPASS; ++p) {
             const int ch = (c + p * LPR) * VEC;
@@ -97,11 +98,6 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) gv[p][e] = 0.0f;
             }
-        }
-#pragma unroll
-        for (int e = 0; e < NE; ++e) {
-            const int ch = c + e * LPR;
-            gs[e] = (unit_ok && ch < a.hd) ? to_f32(grow[ch]) : 0.0f;
         }
 
         for (int c0 = 0; c0 < a.S; c0 += kChunk) {
@@ -130,12 +126,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             }
             wave_lds_sync();
 
-            // ---- gather, dots, scatter ----------------------------------------------------
+            // ---- gather and dots -------------------------------------------------------
             const int ns = (a.S - c0) < kChunk ? (a.S - c0) : kChunk;
             const Entry* mine = stage + g * kChunkStride;
             for (int sl = 0; sl < ns; ++sl) {
                 const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
-                const f32x4 w = *reinterpret_cast<const f32x4*>(mine[sl].w);
                 float d[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int p = 0; p < NPASS; ++p) {
@@ -150,22 +145,42 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
                     }
                 }
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const uint32_t base = (off[k] << GSHIFT) + ghead_off;
-#pragma unroll
-                    for (int e = 0; e < NE; ++e) {
-                        const int ch = c + e * LPR;
-                        if (ch < a.hd)
-                            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[k] * gs[e], gres, base + ch * 4u, 0, 0);
-                    }
-                }
                 f32x4 dsum;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) dsum[k] = group_sum(d[k], lpr_log2);
                 if (c == 0) dots[g * kChunk + sl] = dsum;
             }
             wave_lds_sync();
+            // ---- scatter: grad_value[row_c] += (w_c*attn) * grad_out row --------------------
+            // `span` consecutive lanes own consecutive floats of one row, so every atomic
+            // instruction covers 64/span rows with fully contiguous 64-byte pieces: the
+            // atomics are carried out at the memory side at a fixed rate per 64-byte request,
+            // whatever part of the 64 bytes a request uses.
+            {
+                const int nsub = kWave >> span_log2;
+                const int sub = lane >> span_log2, ch0 = lane & ((1 << span_log2) - 1);
+                for (int u = sub; u < U; u += nsub) {
+                    const int qq = q0 + u;
+                    if (qq >= wk.q_end) break;  // later units of this lane are past the end too
+                    const T* gr = gout + (((int64_t)wk.b * a.nq + qq) * a.nh + wk.h) * a.hd;
+                    const Entry* ent = stage + u * kChunkStride;
+                    for (int chb = 0; chb < a.hd; chb += (1 << span_log2)) {
+                        const int ch = chb + ch0;
+                        if (ch < a.hd) {
+                            const float gg = to_f32(gr[ch]);
+                            const uint32_t choff_g = ghead_off + (uint32_t)ch * 4u;
+                            for (int sl = 0; sl < ns; ++sl) {
+                                const u32x4 off = *reinterpret_cast<const u32x4*>(ent[sl].off);
+                                const f32x4 w = *reinterpret_cast<const f32x4*>(ent[sl].w);
+#pragma unroll
+                                for (int k = 0; k < 4; ++k)
+                                    __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(w[k] * gg, gres,
+                                                                                    (off[k] << GSHIFT) + choff_g, 0, 0);
+                            }
+                        }
+                    }
+                }
+            }
 
             // ---- grad_attn / grad_loc from the reduced dots, one sample per lane ----------
             for (int i = lane; i < entries; i += kWave) {
