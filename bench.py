@@ -54,8 +54,8 @@ def _kernel_times(d, iters, warmup):
     _, nq, _, nl, npts, _ = d.sampling_locations.shape
     out = torch.empty(bs, nq, nh * hd, dtype=dt, device=d.value.device)
     gv, gl, ga = torch.zeros_like(d.value), torch.empty_like(d.sampling_locations), torch.empty_like(d.attention_weights)
-    ws_bytes = lib.mxd_msda_backward_workspace_bytes(code, bs, nk, nh, hd)
-    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=d.value.device)
+    ws_bytes = lib.mxd_msda_backward_workspace_bytes(code, bs, nk, nh, hd, nl, nl, nq, npts)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=d.value.device)
     stream = torch.cuda.current_stream().cuda_stream
     dims = (bs, nk, nh, hd, nl, nl, nq, npts)
 
@@ -69,7 +69,7 @@ def _kernel_times(d, iters, warmup):
         rc = lib.mxd_msda_backward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(),
                                    d.sampling_locations.data_ptr(), d.attention_weights.data_ptr(),
                                    d.grad_output.data_ptr(), gv.data_ptr(), gl.data_ptr(), ga.data_ptr(),
-                                   ws.data_ptr() if ws_bytes else None, ws_bytes, code, *dims, flags, stream)
+                                   ws.data_ptr(), ws_bytes, code, *dims, flags, stream)
         assert rc == 0, _lib.last_error()
 
     res = {"forward_ms": _event_ms(fwd, iters, warmup), "backward_with_zero_fill_ms": _event_ms(lambda: bwd(0), iters, warmup)}

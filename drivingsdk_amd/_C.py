@@ -102,13 +102,13 @@ def multi_scale_deformable_attn_backward(value, shape, level_start_index, locati
     grad_loc = torch.empty_like(loc)
     grad_attn = torch.empty_like(attn)
     code = _FLOAT_CODES[dt]
-    ws_bytes = lib.mxd_msda_backward_workspace_bytes(code, bs, nk, nh, hd)
-    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=value.device) if ws_bytes else None
+    ws_bytes = lib.mxd_msda_backward_workspace_bytes(code, bs, nk, nh, hd, nl, nl_attn, nq, npts)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=value.device)
     with torch.cuda.device(value.device):
         stream = torch.cuda.current_stream().cuda_stream
         rc = lib.mxd_msda_backward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(), attn.data_ptr(),
                                    gout.data_ptr(), grad_value.data_ptr(), grad_loc.data_ptr(), grad_attn.data_ptr(),
-                                   workspace.data_ptr() if workspace is not None else None, ws_bytes, code, bs, nk,
+                                   workspace.data_ptr(), ws_bytes, code, bs, nk,
                                    nh, hd, nl, nl_attn, nq, npts, 0, stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return grad_value, grad_loc, grad_attn

@@ -63,7 +63,7 @@ def load():
     lib.mxd_msda_forward.restype = ci
     lib.mxd_msda_forward.argtypes = [p] * 6 + [ci] + [i64] * 8 + [p]
     lib.mxd_msda_backward_workspace_bytes.restype = ctypes.c_size_t
-    lib.mxd_msda_backward_workspace_bytes.argtypes = [ci] + [i64] * 4
+    lib.mxd_msda_backward_workspace_bytes.argtypes = [ci] + [i64] * 8
     lib.mxd_msda_backward.restype = ci
     lib.mxd_msda_backward.argtypes = [p] * 10 + [ctypes.c_size_t, ci] + [i64] * 8 + [ci, p]
     _lib = lib

@@ -22,7 +22,7 @@
 
 namespace mxd {
 
-template <typename T, int VEC, int NPASS>
+template <typename T, int VEC, int NPASS, bool SCATTER>
 __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
     constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             // instruction covers 64/span rows with fully contiguous 64-byte pieces: the
             // atomics are carried out at the memory side at a fixed rate per 64-byte request,
             // whatever part of the 64 bytes a request uses.
-            {
+            if constexpr (SCATTER) {
                 const int nsub = kWave >> span_log2;
                 const int sub = lane >> span_log2, ch0 = lane & ((1 << span_log2) - 1);
                 for (int u = sub; u < U; u += nsub) {
@@ -204,6 +204,12 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     gattn[e] = from_f32<T>(ga);
                     gloc[2 * e] = from_f32<T>(gx);
                     gloc[2 * e + 1] = from_f32<T>(gy);
+                    if constexpr (!SCATTER) {
+                        // level-major key for the tile kernel: pixel index of the (y0, x0) corner
+                        const int p = s - l * a.np;
+                        a.keys[((((int64_t)wk.b * a.nh + wk.h) * a.nl + l) * a.nq + q) * a.np + p] =
+                            sm.valid ? sm.pix[0] : INT32_MIN;
+                    }
                 }
             }
             wave_lds_sync();
@@ -277,35 +283,41 @@ hipError_t launch_round(int dtype, const float* src, void* dst, size_t n, hipStr
 }
 
 template <typename T, int VEC, int NPASS>
-static hipError_t launch_one(const KArgs& a, hipStream_t stream)
+static hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
 {
-    hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS>), dim3(a.plan.grid), dim3(a.plan.block), a.plan.lds_bytes,
-                       stream, a);
+    if (scatter)
+        hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true>), dim3(a.plan.grid), dim3(a.plan.block),
+                           a.plan.lds_bytes, stream, a);
+    else
+        hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false>), dim3(a.plan.grid), dim3(a.plan.block),
+                           a.plan.lds_bytes, stream, a);
     return hipGetLastError();
 }
 
 template <typename T>
-static hipError_t launch_dtype(const KArgs& a, hipStream_t stream)
+static hipError_t launch_dtype(const KArgs& a, bool scatter, hipStream_t stream)
 {
     const int vec = a.plan.vec, np = a.plan.npass;
-    if (vec == 1 && np == 1) return launch_one<T, 1, 1>(a, stream);
-    if (vec == 1 && np == 2) return launch_one<T, 1, 2>(a, stream);
-    if (vec == 1 && np == 4) return launch_one<T, 1, 4>(a, stream);
-    if (vec == 2 && np == 1) return launch_one<T, 2, 1>(a, stream);
-    if (vec == 2 && np == 2) return launch_one<T, 2, 2>(a, stream);
-    if (vec == 4 && np == 1) return launch_one<T, 4, 1>(a, stream);
+    if (vec == 1 && np == 1) return launch_one<T, 1, 1>(a, scatter, stream);
+    if (vec == 1 && np == 2) return launch_one<T, 1, 2>(a, scatter, stream);
+    if (vec == 1 && np == 4) return launch_one<T, 1, 4>(a, scatter, stream);
+    if (vec == 2 && np == 1) return launch_one<T, 2, 1>(a, scatter, stream);
+    if (vec == 2 && np == 2) return launch_one<T, 2, 2>(a, scatter, stream);
+    if (vec == 4 && np == 1) return launch_one<T, 4, 1>(a, scatter, stream);
     if constexpr (sizeof(T) == 2) {
-        if (vec == 8 && np == 1) return launch_one<T, 8, 1>(a, stream);
+        if (vec == 8 && np == 1) return launch_one<T, 8, 1>(a, scatter, stream);
     }
     return hipErrorInvalidConfiguration;
 }
 
-hipError_t launch_backward(int dtype, const KArgs& a, hipStream_t stream)
+// scatter = true: one kernel does everything (grad_value through global atomics);
+// scatter = false: grad_attn / grad_loc only, grad_value is left to the tile kernel.
+hipError_t launch_backward(int dtype, const KArgs& a, bool scatter, hipStream_t stream)
 {
     switch (dtype) {
-        case MXD_DTYPE_F32: return launch_dtype<float>(a, stream);
-        case MXD_DTYPE_F16: return launch_dtype<f16_t>(a, stream);
-        case MXD_DTYPE_BF16: return launch_dtype<bf16_t>(a, stream);
+        case MXD_DTYPE_F32: return launch_dtype<float>(a, scatter, stream);
+        case MXD_DTYPE_F16: return launch_dtype<f16_t>(a, scatter, stream);
+        case MXD_DTYPE_BF16: return launch_dtype<bf16_t>(a, scatter, stream);
         default: return hipErrorInvalidValue;
     }
 }

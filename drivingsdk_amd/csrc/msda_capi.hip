@@ -10,7 +10,8 @@
 
 namespace mxd {
 hipError_t launch_forward(int dtype, const KArgs& a, hipStream_t stream);
-hipError_t launch_backward(int dtype, const KArgs& a, hipStream_t stream);
+hipError_t launch_backward(int dtype, const KArgs& a, bool scatter, hipStream_t stream);
+hipError_t launch_gradv_tiles(int dtype, const KArgs& a, const TileArgs& t, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t stream);
 hipError_t launch_round(int dtype, const float* src, void* dst, size_t n, hipStream_t stream);
 }  // namespace mxd
@@ -71,6 +72,57 @@ int check_dims(int dtype, const Dims& d)
     return MXD_OK;
 }
 
+// Fills the XCD mapping fields of a plan for `ntiles` work items per (batch, head); returns the grid.
+int64_t fill_xcd_map(mxd_msda_plan* p, int64_t bs, int64_t nh, int64_t ntiles)
+{
+    p->ntiles = (int32_t)ntiles;
+    const int mode_override = env_int("MXD_MSDA_XCD_MODE", -1);
+    if (mode_override != 0 && nh % mxd::kNumXcd == 0) {
+        p->xcd_mode = 1;
+        p->heads_per_xcd = (int32_t)(nh / mxd::kNumXcd);
+        p->xcds_per_head = 1;
+        p->tiles_per_part = (int32_t)ntiles;
+        return (int64_t)mxd::kNumXcd * p->heads_per_xcd * ntiles * bs;
+    }
+    if (mode_override != 0 && mxd::kNumXcd % nh == 0) {
+        p->xcd_mode = 2;
+        p->heads_per_xcd = 1;
+        p->xcds_per_head = (int32_t)(mxd::kNumXcd / nh);
+        p->tiles_per_part = (int32_t)((ntiles + p->xcds_per_head - 1) / p->xcds_per_head);
+        return (int64_t)mxd::kNumXcd * p->tiles_per_part * bs;
+    }
+    p->xcd_mode = 0;
+    p->heads_per_xcd = 1;
+    p->xcds_per_head = 1;
+    p->tiles_per_part = (int32_t)ntiles;
+    return bs * nh * ntiles;
+}
+
+// Geometry of the tile-ownership grad_value kernel (msda_bwd_tiles.hip).
+int make_tile_args(const Dims& d, int vec, int accumulate, mxd::TileArgs* t)
+{
+    memset(t, 0, sizeof(*t));
+    int64_t tile_px = mxd::kTilePx;
+    if (tile_px > d.nk) tile_px = d.nk;
+    t->tile_px = (int32_t)tile_px;
+    t->target = env_int("MXD_MSDA_TILE_TARGET", 4096);
+    if (t->target < 64) t->target = 64;
+    t->max_chunks = 64;
+    // work items per (batch, head): sum over levels of tiles*chunks <= nl*nq*np/target + sum of tiles,
+    // and a level has at most nk/tile_px + 1 tiles whatever spatial_shapes says
+    const int64_t items = (d.nl * d.nq * d.np + t->target - 1) / t->target + d.nl * (d.nk / tile_px + 1);
+    if (items >= (int64_t(1) << 24)) return fail(MXD_E_SHAPE, "backward needs %lld work items per (batch, head)", (long long)items);
+    t->items_per_bh = (int32_t)items;
+    t->vec = vec;
+    t->accumulate = accumulate;
+    t->map.tile_q = 1;
+    const int64_t grid = fill_xcd_map(&t->map, d.bs, d.nh, items);
+    if (grid >= (int64_t(1) << 31)) return fail(MXD_E_SHAPE, "backward needs %lld workgroups, beyond the launch limit", (long long)grid);
+    t->grid = (uint32_t)grid;
+    t->block = mxd::kTilePx;
+    return MXD_OK;
+}
+
 int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_plan* p)
 {
     const int rc = check_dims(dtype, d);
@@ -96,27 +148,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     p->tile_q = p->units_per_wave * p->waves_per_block * p->iters;
     const int64_t ntiles = (d.nq + p->tile_q - 1) / p->tile_q;
     p->ntiles = (int32_t)ntiles;
-    int64_t grid;
-    const int mode_override = env_int("MXD_MSDA_XCD_MODE", -1);
-    if (mode_override != 0 && d.nh % mxd::kNumXcd == 0) {
-        p->xcd_mode = 1;
-        p->heads_per_xcd = (int32_t)(d.nh / mxd::kNumXcd);
-        p->xcds_per_head = 1;
-        p->tiles_per_part = (int32_t)ntiles;
-        grid = (int64_t)mxd::kNumXcd * p->heads_per_xcd * ntiles * d.bs;
-    } else if (mode_override != 0 && mxd::kNumXcd % d.nh == 0) {
-        p->xcd_mode = 2;
-        p->heads_per_xcd = 1;
-        p->xcds_per_head = (int32_t)(mxd::kNumXcd / d.nh);
-        p->tiles_per_part = (int32_t)((ntiles + p->xcds_per_head - 1) / p->xcds_per_head);
-        grid = (int64_t)mxd::kNumXcd * p->tiles_per_part * d.bs;
-    } else {
-        p->xcd_mode = 0;
-        p->heads_per_xcd = 1;
-        p->xcds_per_head = 1;
-        p->tiles_per_part = (int32_t)ntiles;
-        grid = d.bs * d.nh * ntiles;
-    }
+    const int64_t grid = fill_xcd_map(p, d.bs, d.nh, ntiles);
     if (grid >= (int64_t(1) << 31)) return fail(MXD_E_SHAPE, "problem needs %lld workgroups, beyond the launch limit", (long long)grid);
     p->grid = (uint32_t)grid;
     p->block = (uint32_t)(p->waves_per_block * mxd::kWave);
@@ -208,10 +240,21 @@ int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int
     return MXD_OK;
 }
 
-size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd)
+// workspace layout: [keys: bs*nh*nl*nq*np int32, padded to 256 B][fp32 image of grad_value, 16-bit dtypes only]
+static size_t keys_bytes(const Dims& d)
 {
-    if (elem_size(dtype) != 2 || bs <= 0 || nk <= 0 || nh <= 0 || hd <= 0) return 0;
-    return (size_t)bs * (size_t)nk * (size_t)nh * (size_t)hd * 4;
+    const size_t n = (size_t)d.bs * d.nh * d.nl * d.nq * d.np * 4;
+    return (n + 255) & ~(size_t)255;
+}
+
+size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
+                                         int64_t nl_attn, int64_t nq, int64_t np)
+{
+    const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
+    if (check_dims(dtype, d) != MXD_OK) return 0;
+    size_t n = keys_bytes(d);
+    if (elem_size(dtype) == 2) n += (size_t)bs * nk * nh * hd * 4;
+    return n;
 }
 
 int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
@@ -226,14 +269,19 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !grad_output || !grad_value ||
         !grad_loc || !grad_attn)
         return fail(MXD_E_NULL, "mxd_msda_backward: NULL data pointer");
-    const size_t need = mxd_msda_backward_workspace_bytes(dtype, bs, nk, nh, hd);
-    if (need > 0 && (!workspace || workspace_bytes < need))
+    const size_t need = mxd_msda_backward_workspace_bytes(dtype, bs, nk, nh, hd, nl, nl_attn, nq, np);
+    if (!workspace || workspace_bytes < need)
         return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace of %zu bytes required, %zu given", need,
                     workspace ? workspace_bytes : (size_t)0);
-    if ((flags & MXD_BWD_ACCUMULATE) && need > 0)
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u)
+        return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace must be 16-byte aligned");
+    const bool half = elem_size(dtype) == 2;
+    if ((flags & MXD_BWD_ACCUMULATE) && half)
         return fail(MXD_E_DTYPE, "mxd_msda_backward: MXD_BWD_ACCUMULATE is only available for float32");
-    float* image = need > 0 ? static_cast<float*>(workspace) : static_cast<float*>(grad_value);
-    if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_msda_backward: grad image is not 4-byte aligned");
+    int32_t* keys = static_cast<int32_t*>(workspace);
+    float* image = half ? reinterpret_cast<float*>(static_cast<char*>(workspace) + keys_bytes(d))
+                        : static_cast<float*>(grad_value);
+    if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_msda_backward: grad_value is not 4-byte aligned");
     int align = ptr_align(value);
     if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
     mxd::KArgs a;
@@ -248,6 +296,7 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     a.attn = attn_weight;
     a.grad_out = grad_output;
     a.grad_value = image;
+    a.keys = keys;
     a.grad_loc = grad_loc;
     a.grad_attn = grad_attn;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
@@ -255,9 +304,17 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     hipError_t e = hipSuccess;
     if (!(flags & MXD_BWD_ACCUMULATE)) e = mxd::launch_fill_zero(image, n, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: zero-fill launch failed: %s", hipGetErrorString(e));
-    e = mxd::launch_backward(dtype, a, stream);
+    const bool atomic_mode = env_int("MXD_MSDA_BWD_ATOMIC", 0) != 0;
+    e = mxd::launch_backward(dtype, a, atomic_mode, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: launch failed: %s", hipGetErrorString(e));
-    if (need > 0) {
+    if (!atomic_mode) {
+        mxd::TileArgs t;
+        rc = make_tile_args(d, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
+        if (rc != MXD_OK) return rc;
+        e = mxd::launch_gradv_tiles(dtype, a, t, stream);
+        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: tile kernel launch failed: %s", hipGetErrorString(e));
+    }
+    if (half) {
         e = mxd::launch_round(dtype, image, grad_value, n, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: rounding launch failed: %s", hipGetErrorString(e));
     }

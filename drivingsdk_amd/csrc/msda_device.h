@@ -28,6 +28,7 @@ struct KArgs {
     float* grad_value;     // fp32 accumulation image of grad_value
     void* grad_loc;
     void* grad_attn;
+    int32_t* keys;         // [bs, nh, nl, nq, np] pixel index of each sample's top-left corner (INT32_MIN: invalid)
     int32_t bs, nk, nh, hd, nl, np, nq;
     int32_t S;             // nl*np: samples per unit that are evaluated
     int32_t S_full;        // nl_attn*np: samples per unit that are stored
@@ -36,6 +37,20 @@ struct KArgs {
     uint32_t batch_bytes;  // nk*pitch_bytes
     uint32_t gbatch_bytes; // nk*nh*hd*4: one batch element of the fp32 grad image
     mxd_msda_plan plan;
+};
+
+// Launch description of the tile-ownership grad_value kernel.
+constexpr int kTilePx = 512;      // pixels per tile = threads per workgroup (a lane owns a pixel)
+constexpr int kTileEntCap = 512;  // list entries per wavefront and round
+struct TileArgs {
+    mxd_msda_plan map;     // only the XCD mapping fields are used: one "query" per work item
+    int32_t tile_px;       // pixels per tile at most (<= kTilePx)
+    int32_t target;        // samples per work item aimed at when a hot tile is split by query range
+    int32_t max_chunks;    // most query chunks a tile is split into
+    int32_t items_per_bh;  // upper bound of work items per (batch, head)
+    int32_t vec;           // elements per load of a grad_out row
+    int32_t accumulate;    // add into the existing contents of the image
+    uint32_t grid, block;
 };
 
 // One staged sample: byte offsets of its four corner rows inside the batch element's value

@@ -115,10 +115,14 @@ int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int
                      int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
                      void* hip_stream);
 
-/* Bytes of scratch mxd_msda_backward needs: 0 for fp32; for fp16/bf16 an fp32 image of
- * grad_value (bs*nk*nh*hd*4) that the scatter accumulates into before one rounding pass
- * (the reference keeps the same fp32 buffer, MultiScaleDeformableAttn.cpp:93,103-113). */
-size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd);
+/* Bytes of scratch mxd_msda_backward needs (0 if the sizes are invalid).  It holds one int32
+ * key per sample (bs*nh*nl*nq*np*4 bytes, the pixel index of the sample's top-left corner,
+ * written by the first backward kernel and scanned by the second) and, for fp16/bf16, an fp32
+ * image of grad_value (bs*nk*nh*hd*4) that the sums are formed in before one rounding pass
+ * (the reference keeps the same fp32 buffer, MultiScaleDeformableAttn.cpp:93,103-113; its
+ * launcher also allocates a workspace per call, include/csrc/OpApiCommon.h:589-595). */
+size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
+                                         int64_t nl_attn, int64_t nq, int64_t np);
 
 /* flags of mxd_msda_backward */
 #define MXD_BWD_ACCUMULATE 1 /* fp32 only: add into the caller's grad_value instead of zero-filling it
@@ -127,9 +131,9 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
 /* Backward.  Replaces multi_scale_deformable_attn_backward
  * (mx_driving/csrc/MultiScaleDeformableAttn.cpp:68-118).  On `hip_stream`, in order:
  * zero-fills the fp32 accumulation image of grad_value (grad_value itself for fp32, the
- * workspace otherwise; skipped under MXD_BWD_ACCUMULATE), runs the scatter/reduction kernel,
- * and for fp16/bf16 rounds the workspace into grad_value.  Every element of the three
- * outputs is written. */
+ * workspace otherwise; skipped under MXD_BWD_ACCUMULATE), runs the gradient kernels, and for
+ * fp16/bf16 rounds the image into grad_value.  Every element of the three outputs is written.
+ * `workspace` (16-byte aligned, at least mxd_msda_backward_workspace_bytes()) is required. */
 int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
                       const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
                       void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype,

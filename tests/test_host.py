@@ -103,9 +103,12 @@ def test_c_abi_rejects_bad_sizes(dims, fragment):
 
 def test_workspace_size():
     lib = _lib.load()
-    assert lib.mxd_msda_backward_workspace_bytes(0, 2, 100, 8, 32) == 0
-    assert lib.mxd_msda_backward_workspace_bytes(1, 2, 100, 8, 32) == 2 * 100 * 8 * 32 * 4
-    assert lib.mxd_msda_backward_workspace_bytes(2, 2, 100, 8, 32) == 2 * 100 * 8 * 32 * 4
+    keys = 2 * 8 * 4 * 50 * 3 * 4  # bs*nh*nl*nq*np int32, already a multiple of 256
+    assert keys % 256 == 0
+    assert lib.mxd_msda_backward_workspace_bytes(0, 2, 100, 8, 32, 4, 4, 50, 3) == keys
+    assert lib.mxd_msda_backward_workspace_bytes(1, 2, 100, 8, 32, 4, 4, 50, 3) == keys + 2 * 100 * 8 * 32 * 4
+    assert lib.mxd_msda_backward_workspace_bytes(2, 2, 100, 8, 32, 4, 4, 50, 3) == keys + 2 * 100 * 8 * 32 * 4
+    assert lib.mxd_msda_backward_workspace_bytes(0, 2, 100, 8, 300, 4, 4, 50, 3) == 0  # invalid sizes
 
 
 def _cpu_inputs(dtype=torch.float32):
