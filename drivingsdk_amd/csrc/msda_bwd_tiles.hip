@@ -11,19 +11,20 @@
 // registers are fast, so the scatter is turned inside out:
 //
 //   * The pixels of every level are cut into tiles of kTilePx pixels.  A workgroup owns one
-//     tile of one (batch, head); LANE i OWNS PIXEL i of the tile and keeps that pixel's
-//     channels in registers for the whole kernel.
+//     tile of one (batch, head); every group of 4 lanes owns 4 pixels of the tile and keeps
+//     their channels in registers for the whole kernel.
 //   * The backward's first kernel leaves, per sample, the pixel index of its top-left corner
 //     in a level-major key array.  The owner scans the keys of its (batch, head, level) --
 //     4 contiguous bytes per sample -- and rejects samples that cannot touch the tile with
-//     two compares.  For the rest it recomputes the geometry and, per corner inside the
-//     tile, appends an entry {query, weight} to that PIXEL's linked list in LDS (one integer
-//     exchange on the list head; entry storage is private to the wavefront, so no allocation
-//     atomics are needed).
+//     two compares.  Survivors are compacted (ballot + prefix) so that the geometry runs on
+//     dense batches of 64; per corner inside the tile an entry {query, weight} is appended to
+//     that PIXEL's linked list in LDS (one integer exchange on the list head; entry storage
+//     is private to the wavefront, so no allocation atomics are needed).
 //   * When the entry storage fills up (or the scan ends) the workgroup meets at a barrier and
-//     every lane walks its own pixel's list: fetch the grad_out row of the entry's query,
-//     fma into the registers.  No atomics, no read-modify-write of shared accumulators.
-//   * At the end each wavefront transposes its registers through LDS and writes whole rows:
+//     every lane group walks the lists of its own pixels: coalesced 16-byte loads of the
+//     grad_out row of the entry's query, fma into the registers.  No atomics, no
+//     read-modify-write of shared accumulators.
+//   * At the end each wavefront passes its registers through LDS and writes whole rows:
 //     plain stores for tiles a single workgroup owns, a few atomics per workgroup for tiles of
 //     hot (coarse) levels, which are split over several workgroups by query range.
 //
@@ -35,6 +36,9 @@
 namespace mxd {
 
 constexpr uint32_t kNil = 0xFFFFFFFFu;
+constexpr int kLpp = 4;                                  // lanes per pixel row = pixels per lane group
+constexpr int kScanBlocks = 4;                           // blocks of 64 keys fetched together
+constexpr int kCandCap = kWave + kScanBlocks * kWave;    // accepted candidates a wavefront can hold
 
 // Work item table, evaluated identically by every workgroup.
 struct TileItem {
@@ -83,13 +87,17 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
 // CH = channels a lane accumulates per pass (registers); heads with more channels are done in
 // several passes over the same candidates.  VEC = elements per load of a grad_out row.
 template <typename T, int CH, int VEC>
-__global__ __launch_bounds__(kTilePx) void msda_gradv_tiles_kernel(const KArgs a, const TileArgs t)
+__global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArgs a, const TileArgs t)
 {
+    constexpr int CHL = CH / kLpp;                      // channels per lane
+    constexpr int NPC = CHL / 4;                        // 4-channel pieces per lane
+    static_assert(CH % (4 * kLpp) == 0 && 4 % VEC == 0, "a lane owns whole 4-channel pieces");
     constexpr int NW = kTilePx / kWave;                 // wavefronts per workgroup
     __shared__ uint32_t heads[kTilePx];                 // list head per pixel (entry index or kNil)
-    __shared__ uint32_t ent_q[NW * kTileEntCap];        // entry: query index
+    __shared__ uint32_t ent_g[NW * kTileEntCap];        // entry: byte offset of the grad_out row
     __shared__ float ent_w[NW * kTileEntCap];           //        weight
     __shared__ uint32_t ent_next[NW * kTileEntCap];     //        next entry of the same pixel
+    __shared__ uint32_t cq_all[NW * kCandCap];          // accepted candidate indices, per wavefront
     __shared__ TileItem item_s;
     __shared__ int item_ok;
     __shared__ int done_count;
@@ -111,6 +119,7 @@ __global__ __launch_bounds__(kTilePx) void msda_gradv_tiles_kernel(const KArgs a
     const int wave = tid >> 6;
     const int npx = it.p1 - it.p0;
     const uint32_t seg = wave * kTileEntCap;  // this wavefront's entry storage
+    uint32_t* cq = cq_all + wave * kCandCap;
 
     const T* loc = static_cast<const T*>(a.loc);
     const T* attn = static_cast<const T*>(a.attn);
@@ -132,35 +141,78 @@ __global__ __launch_bounds__(kTilePx) void msda_gradv_tiles_kernel(const KArgs a
     float* gimg = a.grad_value + (size_t)wk.b * (a.gbatch_bytes / 4);
     const int64_t row_pitch = (int64_t)a.nh * hd;  // floats between neighbouring pixels
     // transposition scratch of this wavefront (aliases its entry storage; used only after the last round)
-    float* tr = reinterpret_cast<float*>(&ent_q[seg]);
+    float* tr = &ent_w[seg];
+    const uint32_t row_bytes = (uint32_t)(a.nh * hd * (int)sizeof(T));  // between the grad_out rows of two queries
+    // grad_out of this batch element as a bound buffer: offsets >= 2^31 read as zeros
+    const uint32_t gout_batch_bytes = (uint32_t)a.nq * row_bytes;
+    const __amdgpu_buffer_rsrc_t gres =
+        make_rsrc(reinterpret_cast<const char*>(gout) + (size_t)wk.b * gout_batch_bytes, gout_batch_bytes);
+    const uint32_t ghead_off = (uint32_t)wk.h * hd * (uint32_t)sizeof(T);
+    // the last entry slot of every wavefront is its dummy entry
+    const uint32_t dummy = seg + kTileEntCap - 1;
+    if (lane == 0) {
+        ent_g[dummy] = kInvalidCorner;
+        ent_w[dummy] = 0.0f;
+        ent_next[dummy] = kNil;
+    }
 
     for (int cb = 0; cb < hd; cb += CH) {
-        float acc[CH];
+        // lane j of group g = tid/kLpp keeps, for each of the pixels g*kLpp .. g*kLpp+kLpp-1, channels
+        // 4j..4j+3 of every piece of 4*kLpp channels
+        float acc[kLpp][CHL];
 #pragma unroll
-        for (int c = 0; c < CH; ++c) acc[c] = 0.0f;
+        for (int i = 0; i < kLpp; ++i)
+#pragma unroll
+            for (int c = 0; c < CHL; ++c) acc[i][c] = 0.0f;
 
-        int cursor = my_begin;   // wavefront-uniform
-        bool counted = false;    // this wavefront has reported the end of its candidates
+        int cursor = my_begin;   // next unscanned candidate of this wavefront (uniform)
+        int ncq = 0;             // accepted candidates waiting in cq (uniform)
+        bool counted = false;    // this wavefront has reported the end of its work
         while (true) {
-            // ---- scan + append ------------------------------------------------------------
+            // ---- scan keys, compact accepted candidates, append list entries ---------------
             int count = 0;  // entries of this wavefront in this round (uniform)
-            while (cursor < my_end && count + 4 * kWave <= kTileEntCap) {
-                const int idx = cursor + lane;
-                int32_t key = INT32_MIN;
-                if (idx < my_end) key = keys[idx];
-                cursor += kWave;
-                // corners are key, key+1, key+W, key+W+1
-                const bool maybe = (key != INT32_MIN) && ((int64_t)key + it.W + 1 >= it.p0) && (key < it.p1);
+            while (true) {
+                // (1) refill the candidate queue: kScanBlocks blocks of 64 keys in flight at once
+                while (cursor < my_end && ncq < kWave) {
+                    int32_t key[kScanBlocks];
+#pragma unroll
+                    for (int j = 0; j < kScanBlocks; ++j) {
+                        const int idx = cursor + j * kWave + lane;
+                        key[j] = idx < my_end ? __builtin_nontemporal_load(keys + idx) : INT32_MIN;
+                    }
+#pragma unroll
+                    for (int j = 0; j < kScanBlocks; ++j) {
+                        // corners are key, key+1, key+W, key+W+1
+                        const bool maybe =
+                            (key[j] != INT32_MIN) && ((int64_t)key[j] + it.W + 1 >= it.p0) && (key[j] < it.p1);
+                        const uint64_t mask = __ballot(maybe);
+                        if (mask) {
+                            if (maybe)
+                                cq[ncq + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                                                   __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0))] =
+                                    cursor + j * kWave + lane;
+                            ncq += __builtin_popcountll(mask);
+                        }
+                    }
+                    cursor += kScanBlocks * kWave;
+                }
+                // (2) a dense batch of accepted candidates: geometry + list append
+                const bool flush_tail = cursor >= my_end && ncq > 0;
+                if (!(ncq >= kWave || flush_tail)) break;           // nothing left to do
+                if (count + 4 * kWave > kTileEntCap - 1) break;     // entry storage full: next round
+                const int take = ncq < kWave ? ncq : kWave;
+                wave_lds_sync();
                 int lp[4] = {-1, -1, -1, -1};
                 float wv[4] = {0.f, 0.f, 0.f, 0.f};
                 int q = 0;
-                if (maybe) {
+                if (lane < take) {
+                    const int idx = cq[ncq - take + lane];
                     q = idx / a.np;
                     const int p = idx - q * a.np;
                     const int64_t e = (bh_base + (int64_t)q * a.nh) * a.S_full + s_first + p;
-                    const float x = to_f32(loc[2 * e]);
-                    const float y = to_f32(loc[2 * e + 1]);
-                    const float aw = to_f32(attn[e]);
+                    const float x = to_f32(__builtin_nontemporal_load(loc + 2 * e));
+                    const float y = to_f32(__builtin_nontemporal_load(loc + 2 * e + 1));
+                    const float aw = to_f32(__builtin_nontemporal_load(attn + e));
                     const Sample sm = sample_geometry(x, y, level, a.nk, true);
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
@@ -170,6 +222,8 @@ __global__ __launch_bounds__(kTilePx) void msda_gradv_tiles_kernel(const KArgs a
                         }
                     }
                 }
+                ncq -= take;
+                wave_lds_sync();
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const bool push = lp[k] >= 0;
@@ -179,7 +233,7 @@ __global__ __launch_bounds__(kTilePx) void msda_gradv_tiles_kernel(const KArgs a
                             const uint32_t pos = seg + count +
                                                  __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                                                            __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
-                            ent_q[pos] = (uint32_t)q;
+                            ent_g[pos] = (uint32_t)q * row_bytes;
                             ent_w[pos] = wv[k];
                             ent_next[pos] = atomicExch(&heads[lp[k]], pos);
                         }
@@ -187,49 +241,93 @@ __global__ __launch_bounds__(kTilePx) void msda_gradv_tiles_kernel(const KArgs a
                     }
                 }
             }
-            if (cursor >= my_end && !counted) {
+            if (cursor >= my_end && ncq == 0 && !counted) {
                 counted = true;
                 if (lane == 0) atomicAdd(&done_count, 1);
             }
             __syncthreads();
             const bool all_done = done_count == NW;
 
-            // ---- every lane walks the list of its own pixel -------------------------------
-            uint32_t e = heads[tid];
-            heads[tid] = kNil;
-            while (e != kNil) {
-                const uint32_t q = ent_q[e];
-                const float w = ent_w[e];
-                e = ent_next[e];
-                const T* gr = gout + (bh_base + (int64_t)q * a.nh) * hd + cb;
+            // ---- every group of kLpp lanes walks the lists of its kLpp pixels -----------------
+            // The lanes of a group read one grad_out row with coalesced 16-byte buffer loads
+            // (lane j: channels 4j..4j+3 of every 4*kLpp-channel piece).  The loop body is
+            // branch-free: a list that has ended keeps "reading" the wavefront's dummy entry
+            // (weight 0, out-of-range row offset, for which the buffer load returns zeros), the
+            // trip count is the longest list in the wavefront.  Two entries per trip, so that the
+            // row of the next entry is in flight while the fmas of the current one run.
+            {
+                const int grp = tid / kLpp, j = tid % kLpp;
+                uint32_t piece_off[NPC];
 #pragma unroll
-                for (int c = 0; c < CH; c += VEC) {
-                    if (cb + c < hd) {
-                        float g[VEC];
-                        RowIO<T, VEC>::load_global(gr + c, g);
+                for (int p = 0; p < NPC; ++p) {
+                    const int ch = cb + p * (kLpp * 4) + j * 4;
+                    // channels past head_dim re-read channel 0; their sums are never written out
+                    piece_off[p] = ghead_off + (uint32_t)(ch < hd ? ch : 0) * (uint32_t)sizeof(T);
+                }
+                auto fetch = [&](uint32_t& e, float (&g)[CHL], float& w) {
+                    const uint32_t goff = ent_g[e];
+                    w = ent_w[e];
+                    const uint32_t nx = ent_next[e];
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) acc[c + v] = __builtin_fmaf(w, g[v], acc[c + v]);
+                    for (int p = 0; p < NPC; ++p) {
+#pragma unroll
+                        for (int c = 0; c < 4; c += VEC) {
+                            float g1[VEC];
+                            RowIO<T, VEC>::unpack(
+                                RowIO<T, VEC>::load_raw(gres, goff + piece_off[p] + (uint32_t)(c * sizeof(T))), g1);
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) g[p * 4 + c + v] = g1[v];
+                        }
                     }
+                    e = nx == kNil ? dummy : nx;
+                };
+#pragma unroll
+                for (int i = 0; i < kLpp; ++i) {
+                    const int px = grp * kLpp + i;
+                    uint32_t e = heads[px];
+                    if (j == 0) heads[px] = kNil;  // same wavefront: ordered after the read above
+                    e = e == kNil ? dummy : e;
+                    float ga[CHL], gb[CHL], wa, wb;
+                    fetch(e, ga, wa);
+                    while (__ballot(e != dummy)) {
+                        fetch(e, gb, wb);
+#pragma unroll
+                        for (int c = 0; c < CHL; ++c) acc[i][c] = __builtin_fmaf(wa, ga[c], acc[i][c]);
+                        fetch(e, ga, wa);
+#pragma unroll
+                        for (int c = 0; c < CHL; ++c) acc[i][c] = __builtin_fmaf(wb, gb[c], acc[i][c]);
+                    }
+#pragma unroll
+                    for (int c = 0; c < CHL; ++c) acc[i][c] = __builtin_fmaf(wa, ga[c], acc[i][c]);
                 }
             }
             __syncthreads();
             if (all_done) break;
         }
 
-        // ---- write the CH channels of this tile: transpose through LDS, 8 pixels at a time ----
-        constexpr int TP = 8;                  // pixels per transposition step
-        constexpr int TS = CH + 1;             // padded row stride (LDS banks)
-        static_assert(TP * TS <= kTileEntCap, "transposition scratch must fit the entry storage");
+        // ---- write the CH channels of this tile -------------------------------------------
+        // Eight pixels at a time are parked in LDS; the whole wavefront then writes them with
+        // consecutive lanes on consecutive floats (full 64-byte pieces per request).
+        constexpr int TPX = 8;      // pixels per step
+        constexpr int TS = CH + 1;  // padded row stride (LDS banks)
+        static_assert(TPX * TS <= kTileEntCap, "transposition scratch must fit the entry storage");
         const int nch = (hd - cb) < CH ? (hd - cb) : CH;
-        for (int half = 0; half < kWave / TP; ++half) {
+        for (int o = 0; o < kWave / TPX; ++o) {
             wave_lds_sync();
-            if ((lane / TP) == half) {
+            if ((lane / TPX) == o) {
+                // the TPX lanes of this step are TPX/kLpp groups, each holding kLpp pixels
+                const int gl = (lane % TPX) / kLpp, j = lane % kLpp;
 #pragma unroll
-                for (int c = 0; c < CH; ++c) tr[(lane % TP) * TS + c] = acc[c];
+                for (int i = 0; i < kLpp; ++i)
+#pragma unroll
+                    for (int p = 0; p < NPC; ++p)
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+                            tr[(gl * kLpp + i) * TS + p * (kLpp * 4) + j * 4 + c] = acc[i][p * 4 + c];
             }
             wave_lds_sync();
-            const int px_base = wave * kWave + half * TP;
-            for (int i = lane; i < TP * nch; i += kWave) {
+            const int px_base = wave * kWave + o * TPX;
+            for (int i = lane; i < TPX * nch; i += kWave) {
                 const int pl = i / nch, c = i - pl * nch;
                 const int px = px_base + pl;
                 if (px < npx) {
@@ -257,10 +355,12 @@ __global__ __launch_bounds__(kTilePx) void msda_gradv_tiles_kernel(const KArgs a
 template <typename T>
 static hipError_t launch_t(const KArgs& a, const TileArgs& t, hipStream_t stream)
 {
-    // grad_out rows are read with 16-byte loads when head_dim and the pointer allow it
-    constexpr int WIDE = 16 / (int)sizeof(T);
-    if (t.vec == WIDE)
-        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 32, WIDE>), dim3(t.grid), dim3(t.block), 0, stream, a, t);
+    // an octet of lanes reads a 32-channel slice of a grad_out row, 4 channels per lane: one
+    // load per lane when head_dim and the pointer alignment allow it
+    if (t.vec >= 4)
+        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 32, 4>), dim3(t.grid), dim3(t.block), 0, stream, a, t);
+    else if (t.vec == 2)
+        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 32, 2>), dim3(t.grid), dim3(t.block), 0, stream, a, t);
     else
         hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 32, 1>), dim3(t.grid), dim3(t.block), 0, stream, a, t);
     return hipGetLastError();

@@ -113,6 +113,8 @@ int make_tile_args(const Dims& d, int vec, int accumulate, mxd::TileArgs* t)
     const int64_t items = (d.nl * d.nq * d.np + t->target - 1) / t->target + d.nl * (d.nk / tile_px + 1);
     if (items >= (int64_t(1) << 24)) return fail(MXD_E_SHAPE, "backward needs %lld work items per (batch, head)", (long long)items);
     t->items_per_bh = (int32_t)items;
+    if (d.nq * d.nh * d.hd * 4 >= (int64_t(1) << 31))
+        return fail(MXD_E_SHAPE, "one batch element of grad_output (num_queries*num_heads*embed_dims) must stay below 2 GiB at 4 bytes per element");
     t->vec = vec;
     t->accumulate = accumulate;
     t->map.tile_q = 1;
