@@ -37,7 +37,7 @@ namespace mxd {
 
 constexpr uint32_t kNil = 0xFFFFFFFFu;
 constexpr int kLpp = 4;                                  // lanes per pixel row = pixels per lane group
-constexpr int kScanBlocks = 4;                           // blocks of 64 keys fetched together
+constexpr int kScanBlocks = 8;                           // blocks of 64 keys fetched together
 constexpr int kCandCap = kWave + kScanBlocks * kWave;    // accepted candidates a wavefront can hold
 
 // Work item table, evaluated identically by every workgroup.
@@ -166,20 +166,28 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
             for (int c = 0; c < CHL; ++c) acc[i][c] = 0.0f;
 
         int cursor = my_begin;   // next unscanned candidate of this wavefront (uniform)
+        int32_t pre[kScanBlocks];  // keys of the blocks at `cursor`, fetched one step ahead
+        auto load_keys = [&](int base) {
+#pragma unroll
+            for (int j = 0; j < kScanBlocks; ++j) {
+                const int idx = base + j * kWave + lane;
+                pre[j] = idx < my_end ? __builtin_nontemporal_load(keys + idx) : INT32_MIN;
+            }
+        };
+        load_keys(my_begin);
         int ncq = 0;             // accepted candidates waiting in cq (uniform)
         bool counted = false;    // this wavefront has reported the end of its work
         while (true) {
             // ---- scan keys, compact accepted candidates, append list entries ---------------
             int count = 0;  // entries of this wavefront in this round (uniform)
             while (true) {
-                // (1) refill the candidate queue: kScanBlocks blocks of 64 keys in flight at once
+                // (1) refill the candidate queue from the keys fetched one step ahead, and put the
+                // next kScanBlocks blocks of 64 keys in flight before testing the current ones
                 while (cursor < my_end && ncq < kWave) {
                     int32_t key[kScanBlocks];
 #pragma unroll
-                    for (int j = 0; j < kScanBlocks; ++j) {
-                        const int idx = cursor + j * kWave + lane;
-                        key[j] = idx < my_end ? __builtin_nontemporal_load(keys + idx) : INT32_MIN;
-                    }
+                    for (int j = 0; j < kScanBlocks; ++j) key[j] = pre[j];
+                    load_keys(cursor + kScanBlocks * kWave);
 #pragma unroll
                     for (int j = 0; j < kScanBlocks; ++j) {
                         // corners are key, key+1, key+W, key+W+1
