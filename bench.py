@@ -73,12 +73,22 @@ def _kernel_times(d, iters, warmup):
         assert rc == 0, _lib.last_error()
 
     res = {"forward_ms": _event_ms(fwd, iters, warmup), "backward_with_zero_fill_ms": _event_ms(lambda: bwd(0), iters, warmup)}
-    if code == 0:
-        # scatter kernel alone: accumulate into the (already initialised) gradient image
-        res["backward_kernel_ms"] = _event_ms(lambda: bwd(_lib.BWD_ACCUMULATE), iters, warmup)
-    else:
-        res["backward_kernel_ms"] = None
+    # gradient accumulation into an existing image (no zero-fill, owned tiles add instead of store)
+    res["backward_accumulate_ms"] = _event_ms(lambda: bwd(_lib.BWD_ACCUMULATE), iters, warmup) if code == 0 else None
     return res
+
+
+def _committed_traffic(workload, dtype):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
+    kernel of known size) and committed under profiles/; None when no measurement covers this run."""
+    path = os.path.join(ROOT, "profiles", "traffic_detr_encoder_fp32.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        data = json.load(f)
+    if data.get("workload") != workload or data.get("dtype") != dtype:
+        return None
+    return data["kernels"]
 
 
 def _cpu_baseline(inp, max_seconds=25.0):
@@ -118,6 +128,10 @@ def main():
     ap.add_argument("--workload", default="detr_encoder_bwd")
     ap.add_argument("--dtype", default="float32", choices=["float32", "float16", "bfloat16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also run a plain elementwise copy kernel of value's size (reads and writes "
+                         "value.numel()*4 bytes) so that FETCH_SIZE/WRITE_SIZE of a rocprofv3 --pmc run "
+                         "can be scaled by what the same counters read for a copy of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this operator runs on one GPU; --gpus must be 1 (no multi-GPU path exists in this build)",
@@ -144,6 +158,11 @@ def main():
         out = mx_driving.multi_scale_deformable_attn(value, d.spatial_shapes, d.level_start_index, loc, attn)
         out.backward(d.grad_output)
 
+    if args.traffic_calibration:
+        for _ in range(3):
+            torch.mul(d.value, 1.0)  # vectorized_elementwise_kernel: value bytes in, value bytes out
+        torch.cuda.synchronize()
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -161,15 +180,22 @@ def main():
 
     k = _kernel_times(d, iters=max(args.steps, 50), warmup=max(args.warmup, 10))
 
-    def roof(nbytes, ms, kernel):
-        achieved = nbytes / (ms * 1e-3) / 1e9
-        return {"bound": "hbm", "kernel": kernel, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "algorithmic_bytes": nbytes, "kernel_ms": ms}
+    traffic = _committed_traffic(args.workload, args.dtype)
 
-    roof_fwd = roof(bytes_fwd, k["forward_ms"], "msda_fwd_kernel")
-    bwd_ms = k["backward_kernel_ms"] if k["backward_kernel_ms"] is not None else k["backward_with_zero_fill_ms"]
-    roof_bwd = roof(bytes_bwd, bwd_ms, "msda_bwd_kernel")
-    dominant = roof_bwd if bwd_ms >= k["forward_ms"] else roof_fwd
+    def roof(nbytes, ms, kernels):
+        achieved = nbytes / (ms * 1e-3) / 1e9
+        hbm = None
+        if traffic is not None and all(k in traffic for k in kernels):
+            hbm = sum(traffic[k]["hbm_bytes"] for k in kernels)
+        return {"bound": "hbm", "kernel": " + ".join(kernels), "achieved": achieved, "peak": HBM_PEAK_GBPS,
+                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": hbm, "algorithmic_bytes": nbytes,
+                "kernel_ms": ms}
+
+    roof_fwd = roof(bytes_fwd, k["forward_ms"], ["msda_fwd_kernel"])
+    # the backward pass: zero-fill, per-sample dots (grad_attn, grad_loc, keys), grad_value by tile ownership
+    roof_bwd = roof(bytes_bwd, k["backward_with_zero_fill_ms"],
+                    ["msda_fill_zero_kernel", "msda_bwd_kernel", "msda_gradv_tiles_kernel"])
+    dominant = roof_bwd if roof_bwd["kernel_ms"] >= k["forward_ms"] else roof_fwd
 
     cfg = workloads.WORKLOADS[args.workload]
     result = {
