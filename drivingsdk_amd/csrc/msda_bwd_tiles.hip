@@ -35,9 +35,8 @@
 
 namespace mxd {
 
-constexpr uint32_t kNil = 0xFFFFFFFFu;
-constexpr int kLpp = 4;                                  // lanes per pixel row = pixels per lane group
-constexpr int kScanBlocks = 8;                           // blocks of 64 keys fetched together
+constexpr int kLpp = 8;                                  // lanes per pixel row = pixels per lane group
+constexpr int kScanBlocks = 4;                           // blocks of 64 keys fetched together
 constexpr int kCandCap = kWave + kScanBlocks * kWave;    // accepted candidates a wavefront can hold
 
 // Work item table, evaluated identically by every workgroup.
@@ -84,19 +83,19 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
     return false;
 }
 
-// CH = channels a lane accumulates per pass (registers); heads with more channels are done in
-// several passes over the same candidates.  VEC = elements per load of a grad_out row.
+// CH = channels a lane group accumulates per pass (registers); heads with more channels are
+// done in several passes over the same candidates.  VEC = elements per load of a grad_out row.
 template <typename T, int CH, int VEC>
 __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArgs a, const TileArgs t)
 {
     constexpr int CHL = CH / kLpp;                      // channels per lane
-    constexpr int NPC = CHL / 4;                        // 4-channel pieces per lane
-    static_assert(CH % (4 * kLpp) == 0 && 4 % VEC == 0, "a lane owns whole 4-channel pieces");
+    static_assert(CHL == 4 && 4 % VEC == 0, "a lane owns one 4-channel piece of a row");
     constexpr int NW = kTilePx / kWave;                 // wavefronts per workgroup
-    __shared__ uint32_t heads[kTilePx];                 // list head per pixel (entry index or kNil)
-    __shared__ uint32_t ent_g[NW * kTileEntCap];        // entry: byte offset of the grad_out row
-    __shared__ float ent_w[NW * kTileEntCap];           //        weight
-    __shared__ uint32_t ent_next[NW * kTileEntCap];     //        next entry of the same pixel
+    constexpr uint32_t kDummyOfWave = kTileEntCap - 1;  // last entry slot of every wavefront
+    __shared__ uint32_t heads[kTilePx];                 // list head per pixel (entry index)
+    // entry: {byte offset of the grad_out row, weight for the list's pixel, weight for the
+    // next pixel, next entry of the same list}
+    __shared__ u32x4 ent[NW * kTileEntCap];
     __shared__ uint32_t cq_all[NW * kCandCap];          // accepted candidate indices, per wavefront
     __shared__ TileItem item_s;
     __shared__ int item_ok;
@@ -108,7 +107,8 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         item_ok = decode_tile_item(a, t, wk.q_begin, &item_s) ? 1 : 0;
         done_count = 0;
     }
-    heads[threadIdx.x] = kNil;
+    // an empty list points at the dummy entry of the wavefront that owns the pixel
+    heads[threadIdx.x] = (threadIdx.x >> 6) * kTileEntCap + kDummyOfWave;
     __syncthreads();
     if (!item_ok) return;  // uniform
     const TileItem it = item_s;
@@ -140,38 +140,37 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
 
     float* gimg = a.grad_value + (size_t)wk.b * (a.gbatch_bytes / 4);
     const int64_t row_pitch = (int64_t)a.nh * hd;  // floats between neighbouring pixels
-    // transposition scratch of this wavefront (aliases its entry storage; used only after the last round)
-    float* tr = &ent_w[seg];
     const uint32_t row_bytes = (uint32_t)(a.nh * hd * (int)sizeof(T));  // between the grad_out rows of two queries
     // grad_out of this batch element as a bound buffer: offsets >= 2^31 read as zeros
     const uint32_t gout_batch_bytes = (uint32_t)a.nq * row_bytes;
     const __amdgpu_buffer_rsrc_t gres =
         make_rsrc(reinterpret_cast<const char*>(gout) + (size_t)wk.b * gout_batch_bytes, gout_batch_bytes);
     const uint32_t ghead_off = (uint32_t)wk.h * hd * (uint32_t)sizeof(T);
-    // the last entry slot of every wavefront is its dummy entry
-    const uint32_t dummy = seg + kTileEntCap - 1;
-    if (lane == 0) {
-        ent_g[dummy] = kInvalidCorner;
-        ent_w[dummy] = 0.0f;
-        ent_next[dummy] = kNil;
-    }
+    // the dummy entry ends every list of this wavefront's pixels: weight 0, a row offset the
+    // buffer range check answers with zeros (at no cost in the memory pipeline), next = itself
+    const uint32_t dummy = seg + kDummyOfWave;
+    if (lane == 0) ent[dummy] = u32x4{kInvalidCorner, 0u, 0u, dummy};
+
+    // lane j of group g = tid/kLpp keeps channels 4j..4j+3 of the pixels g*kLpp .. g*kLpp+kLpp-1
+    const int grp = tid / kLpp, j = tid % kLpp;
 
     for (int cb = 0; cb < hd; cb += CH) {
-        // lane j of group g = tid/kLpp keeps, for each of the pixels g*kLpp .. g*kLpp+kLpp-1, channels
-        // 4j..4j+3 of every piece of 4*kLpp channels
         float acc[kLpp][CHL];
 #pragma unroll
         for (int i = 0; i < kLpp; ++i)
 #pragma unroll
             for (int c = 0; c < CHL; ++c) acc[i][c] = 0.0f;
+        // channels past head_dim re-read channel 0; their sums are never written out
+        const int my_ch = cb + j * 4;
+        const uint32_t lane_off = ghead_off + (uint32_t)(my_ch < hd ? my_ch : 0) * (uint32_t)sizeof(T);
 
         int cursor = my_begin;   // next unscanned candidate of this wavefront (uniform)
         int32_t pre[kScanBlocks];  // keys of the blocks at `cursor`, fetched one step ahead
         auto load_keys = [&](int base) {
 #pragma unroll
-            for (int j = 0; j < kScanBlocks; ++j) {
-                const int idx = base + j * kWave + lane;
-                pre[j] = idx < my_end ? __builtin_nontemporal_load(keys + idx) : INT32_MIN;
+            for (int jb = 0; jb < kScanBlocks; ++jb) {
+                const int idx = base + jb * kWave + lane;
+                pre[jb] = idx < my_end ? __builtin_nontemporal_load(keys + idx) : INT32_MIN;
             }
         };
         load_keys(my_begin);
@@ -186,19 +185,19 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 while (cursor < my_end && ncq < kWave) {
                     int32_t key[kScanBlocks];
 #pragma unroll
-                    for (int j = 0; j < kScanBlocks; ++j) key[j] = pre[j];
+                    for (int jb = 0; jb < kScanBlocks; ++jb) key[jb] = pre[jb];
                     load_keys(cursor + kScanBlocks * kWave);
 #pragma unroll
-                    for (int j = 0; j < kScanBlocks; ++j) {
+                    for (int jb = 0; jb < kScanBlocks; ++jb) {
                         // corners are key, key+1, key+W, key+W+1
                         const bool maybe =
-                            (key[j] != INT32_MIN) && ((int64_t)key[j] + it.W + 1 >= it.p0) && (key[j] < it.p1);
+                            (key[jb] != INT32_MIN) && ((int64_t)key[jb] + it.W + 1 >= it.p0) && (key[jb] < it.p1);
                         const uint64_t mask = __ballot(maybe);
                         if (mask) {
                             if (maybe)
                                 cq[ncq + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                                                    __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0))] =
-                                    cursor + j * kWave + lane;
+                                    cursor + jb * kWave + lane;
                             ncq += __builtin_popcountll(mask);
                         }
                     }
@@ -206,12 +205,16 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 }
                 // (2) a dense batch of accepted candidates: geometry + list append
                 const bool flush_tail = cursor >= my_end && ncq > 0;
-                if (!(ncq >= kWave || flush_tail)) break;           // nothing left to do
-                if (count + 4 * kWave > kTileEntCap - 1) break;     // entry storage full: next round
+                if (!(ncq >= kWave || flush_tail)) break;                      // nothing left to do
+                if (count + 4 * kWave > (int)kDummyOfWave) break;              // entry storage full: next round
                 const int take = ncq < kWave ? ncq : kWave;
                 wave_lds_sync();
-                int lp[4] = {-1, -1, -1, -1};
-                float wv[4] = {0.f, 0.f, 0.f, 0.f};
+                // A sample touches two pixel pairs (p, p+1): its upper and its lower corners.  A pair
+                // whose pixels belong to the same lane group becomes ONE entry in the list of the left
+                // pixel (the grad_out row is fetched once for both); otherwise each corner inside the
+                // tile gets an entry of its own with no weight for the neighbour.
+                int lst[4] = {-1, -1, -1, -1};   // list (pixel inside the tile) of up to 4 entries
+                float w0[4] = {0.f, 0.f, 0.f, 0.f}, w1[4] = {0.f, 0.f, 0.f, 0.f};
                 int q = 0;
                 if (lane < take) {
                     const int idx = cq[ncq - take + lane];
@@ -223,10 +226,19 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     const float aw = to_f32(__builtin_nontemporal_load(attn + e));
                     const Sample sm = sample_geometry(x, y, level, a.nk, true);
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        if (sm.cvalid[k] && sm.pix[k] >= it.p0 && sm.pix[k] < it.p1) {
-                            lp[k] = sm.pix[k] - it.p0;
-                            wv[k] = sm.w[k] * aw;
+                    for (int r = 0; r < 2; ++r) {
+                        const int pl = sm.pix[2 * r] - it.p0;  // left pixel of the pair, relative to the tile
+                        const bool in_l = sm.cvalid[2 * r] && pl >= 0 && pl < npx;
+                        const bool in_r = sm.cvalid[2 * r + 1] && pl + 1 >= 0 && pl + 1 < npx;
+                        const bool pair = in_l && in_r && (pl % kLpp) != kLpp - 1;
+                        if (in_l) {
+                            lst[2 * r] = pl;
+                            w0[2 * r] = sm.w[2 * r] * aw;
+                            w1[2 * r] = pair ? sm.w[2 * r + 1] * aw : 0.0f;
+                        }
+                        if (in_r && !pair) {
+                            lst[2 * r + 1] = pl + 1;
+                            w0[2 * r + 1] = sm.w[2 * r + 1] * aw;
                         }
                     }
                 }
@@ -234,16 +246,16 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 wave_lds_sync();
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
-                    const bool push = lp[k] >= 0;
+                    const bool push = lst[k] >= 0;
                     const uint64_t mask = __ballot(push);
                     if (mask) {
                         if (push) {
                             const uint32_t pos = seg + count +
                                                  __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                                                            __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
-                            ent_g[pos] = (uint32_t)q * row_bytes;
-                            ent_w[pos] = wv[k];
-                            ent_next[pos] = atomicExch(&heads[lp[k]], pos);
+                            const uint32_t next = atomicExch(&heads[lst[k]], pos);
+                            ent[pos] = u32x4{(uint32_t)q * row_bytes, __builtin_bit_cast(uint32_t, w0[k]),
+                                             __builtin_bit_cast(uint32_t, w1[k]), next};
                         }
                         count += __builtin_popcountll(mask);
                     }
@@ -257,56 +269,65 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
             const bool all_done = done_count == NW;
 
             // ---- every group of kLpp lanes walks the lists of its kLpp pixels -----------------
-            // The lanes of a group read one grad_out row with coalesced 16-byte buffer loads
-            // (lane j: channels 4j..4j+3 of every 4*kLpp-channel piece).  The loop body is
-            // branch-free: a list that has ended keeps "reading" the wavefront's dummy entry
-            // (weight 0, out-of-range row offset, for which the buffer load returns zeros), the
-            // trip count is the longest list in the wavefront.  Two entries per trip, so that the
-            // row of the next entry is in flight while the fmas of the current one run.
+            // The lanes of a group read one grad_out row with ONE coalesced load (lane j: channels
+            // 4j..4j+3): the memory pipeline's cost is per cache line touched by an instruction.
+            // The loop body is branch-free: a list that has ended keeps "reading" the dummy entry.
+            // Two lists are walked together, two entries of each per trip, so that four row loads
+            // are in flight while the fmas of the previous ones run.
             {
-                const int grp = tid / kLpp, j = tid % kLpp;
-                uint32_t piece_off[NPC];
+                auto fetch = [&](uint32_t& e, float (&g)[CHL], float& wa, float& wb) {
+                    const u32x4 en = ent[e];
+                    // (a bit cast applied directly to a vector element picks up element 0: copy first)
+                    const uint32_t ya = en.y, za = en.z;
+                    wa = __builtin_bit_cast(float, ya);
+                    wb = __builtin_bit_cast(float, za);
 #pragma unroll
-                for (int p = 0; p < NPC; ++p) {
-                    const int ch = cb + p * (kLpp * 4) + j * 4;
-                    // channels past head_dim re-read channel 0; their sums are never written out
-                    piece_off[p] = ghead_off + (uint32_t)(ch < hd ? ch : 0) * (uint32_t)sizeof(T);
-                }
-                auto fetch = [&](uint32_t& e, float (&g)[CHL], float& w) {
-                    const uint32_t goff = ent_g[e];
-                    w = ent_w[e];
-                    const uint32_t nx = ent_next[e];
+                    for (int c = 0; c < 4; c += VEC) {
+                        float g1[VEC];
+                        RowIO<T, VEC>::unpack(RowIO<T, VEC>::load_raw(gres, en.x + lane_off + (uint32_t)(c * sizeof(T))), g1);
 #pragma unroll
-                    for (int p = 0; p < NPC; ++p) {
-#pragma unroll
-                        for (int c = 0; c < 4; c += VEC) {
-                            float g1[VEC];
-                            RowIO<T, VEC>::unpack(
-                                RowIO<T, VEC>::load_raw(gres, goff + piece_off[p] + (uint32_t)(c * sizeof(T))), g1);
-#pragma unroll
-                            for (int v = 0; v < VEC; ++v) g[p * 4 + c + v] = g1[v];
-                        }
+                        for (int v = 0; v < VEC; ++v) g[c + v] = g1[v];
                     }
-                    e = nx == kNil ? dummy : nx;
+                    e = en.w;
                 };
 #pragma unroll
-                for (int i = 0; i < kLpp; ++i) {
+                for (int i = 0; i < kLpp; i += 2) {
                     const int px = grp * kLpp + i;
-                    uint32_t e = heads[px];
-                    if (j == 0) heads[px] = kNil;  // same wavefront: ordered after the read above
-                    e = e == kNil ? dummy : e;
-                    float ga[CHL], gb[CHL], wa, wb;
-                    fetch(e, ga, wa);
-                    while (__ballot(e != dummy)) {
-                        fetch(e, gb, wb);
-#pragma unroll
-                        for (int c = 0; c < CHL; ++c) acc[i][c] = __builtin_fmaf(wa, ga[c], acc[i][c]);
-                        fetch(e, ga, wa);
-#pragma unroll
-                        for (int c = 0; c < CHL; ++c) acc[i][c] = __builtin_fmaf(wb, gb[c], acc[i][c]);
+                    uint32_t ea = heads[px], eb = heads[px + 1];
+                    if (j == 0) {  // same wavefront: ordered after the reads above
+                        heads[px] = dummy;
+                        heads[px + 1] = dummy;
                     }
+                    float ga0[CHL], ga1[CHL], gb0[CHL], gb1[CHL];
+                    float ua0, va0, ua1, va1, ub0, vb0, ub1, vb1;
+                    auto fma_a = [&](const float (&g)[CHL], float u, float v) {
 #pragma unroll
-                    for (int c = 0; c < CHL; ++c) acc[i][c] = __builtin_fmaf(wa, ga[c], acc[i][c]);
+                        for (int c = 0; c < CHL; ++c) {
+                            acc[i][c] = __builtin_fmaf(u, g[c], acc[i][c]);
+                            acc[i + 1][c] = __builtin_fmaf(v, g[c], acc[i + 1][c]);
+                        }
+                    };
+                    auto fma_b = [&](const float (&g)[CHL], float u, float v) {
+#pragma unroll
+                        for (int c = 0; c < CHL; ++c) {
+                            acc[i + 1][c] = __builtin_fmaf(u, g[c], acc[i + 1][c]);
+                            if (i + 2 < kLpp) acc[(i + 2) % kLpp][c] = __builtin_fmaf(v, g[c], acc[(i + 2) % kLpp][c]);
+                        }
+                    };
+                    fetch(ea, ga0, ua0, va0);
+                    fetch(eb, gb0, ub0, vb0);
+                    while (__ballot(ea != dummy || eb != dummy)) {
+                        fetch(ea, ga1, ua1, va1);
+                        fetch(eb, gb1, ub1, vb1);
+                        fma_a(ga0, ua0, va0);
+                        fma_b(gb0, ub0, vb0);
+                        fetch(ea, ga0, ua0, va0);
+                        fetch(eb, gb0, ub0, vb0);
+                        fma_a(ga1, ua1, va1);
+                        fma_b(gb1, ub1, vb1);
+                    }
+                    fma_a(ga0, ua0, va0);
+                    fma_b(gb0, ub0, vb0);
                 }
             }
             __syncthreads();
@@ -314,47 +335,68 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         }
 
         // ---- write the CH channels of this tile -------------------------------------------
-        // Eight pixels at a time are parked in LDS; the whole wavefront then writes them with
-        // consecutive lanes on consecutive floats (full 64-byte pieces per request).
-        constexpr int TPX = 8;      // pixels per step
-        constexpr int TS = CH + 1;  // padded row stride (LDS banks)
-        static_assert(TPX * TS <= kTileEntCap, "transposition scratch must fit the entry storage");
         const int nch = (hd - cb) < CH ? (hd - cb) : CH;
-        for (int o = 0; o < kWave / TPX; ++o) {
-            wave_lds_sync();
-            if ((lane / TPX) == o) {
-                // the TPX lanes of this step are TPX/kLpp groups, each holding kLpp pixels
-                const int gl = (lane % TPX) / kLpp, j = lane % kLpp;
+        if (it.exclusive && t.store_vec == 4) {
+            // the lanes of a group hold a whole row of each of their pixels: 16-byte stores
+            if (my_ch < hd) {
 #pragma unroll
-                for (int i = 0; i < kLpp; ++i)
-#pragma unroll
-                    for (int p = 0; p < NPC; ++p)
-#pragma unroll
-                        for (int c = 0; c < 4; ++c)
-                            tr[(gl * kLpp + i) * TS + p * (kLpp * 4) + j * 4 + c] = acc[i][p * 4 + c];
-            }
-            wave_lds_sync();
-            const int px_base = wave * kWave + o * TPX;
-            for (int i = lane; i < TPX * nch; i += kWave) {
-                const int pl = i / nch, c = i - pl * nch;
-                const int px = px_base + pl;
-                if (px < npx) {
-                    const float v = tr[pl * TS + c];
-                    float* dst = gimg + (int64_t)(it.p0 + px) * row_pitch + (int64_t)wk.h * hd + cb + c;
-                    if (it.exclusive && !t.accumulate)
+                for (int i = 0; i < kLpp; ++i) {
+                    const int px = grp * kLpp + i;
+                    if (px < npx) {
+                        f32x4* dst = reinterpret_cast<f32x4*>(gimg + (int64_t)(it.p0 + px) * row_pitch +
+                                                              (int64_t)wk.h * hd + my_ch);
+                        f32x4 v = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+                        if (t.accumulate) v += *dst;
                         *dst = v;
-                    else if (it.exclusive)
-                        *dst += v;
-                    else
-                        unsafeAtomicAdd(dst, v);
+                    }
                 }
             }
+        } else {
+            // Rows shared with other workgroups (tiles split by query range) are added with
+            // atomics, which the memory side carries out per 64-byte request: pass the registers
+            // through LDS (the entry storage, free after the last round) so that consecutive
+            // lanes hold consecutive floats of a row.  32 pixels at a time.
+            typedef uint32_t __attribute__((may_alias)) u32_alias;
+            static_assert(32 * CH * 4 <= kTileEntCap * 16, "transposition scratch must fit the entry storage");
+            u32x4* tr4 = &ent[seg];
+            const u32_alias* tr1 = reinterpret_cast<const u32_alias*>(tr4);
+            for (int half = 0; half < 2; ++half) {
+                wave_lds_sync();
+                if (((lane / kLpp) >> 2) == half) {
+                    const int gl = (lane / kLpp) & 3;
+#pragma unroll
+                    for (int i = 0; i < kLpp; ++i)
+                        tr4[(gl * kLpp + i) * (CH / 4) + j] =
+                            u32x4{__builtin_bit_cast(uint32_t, acc[i][0]), __builtin_bit_cast(uint32_t, acc[i][1]),
+                                  __builtin_bit_cast(uint32_t, acc[i][2]), __builtin_bit_cast(uint32_t, acc[i][3])};
+                }
+                wave_lds_sync();
+                const int px_base = wave * kWave + half * 32;
+#pragma unroll 4
+                for (int k = 0; k < 32 * CH / kWave; ++k) {
+                    const int idx = k * kWave + lane;
+                    const int pl = idx / CH, c = idx % CH;
+                    const int px = px_base + pl;
+                    if (px < npx && c < nch) {
+                        const float v = __builtin_bit_cast(float, (uint32_t)tr1[idx]);
+                        float* dst = gimg + (int64_t)(it.p0 + px) * row_pitch + (int64_t)wk.h * hd + cb + c;
+                        if (!it.exclusive)
+                            unsafeAtomicAdd(dst, v);
+                        else if (t.accumulate)
+                            *dst += v;
+                        else
+                            *dst = v;
+                    }
+                }
+            }
+            wave_lds_sync();
         }
-        wave_lds_sync();
         if (cb + CH < hd) {
-            // next channel pass starts from a clean state
+            // next channel pass starts from a clean state (the dummy entry may have been
+            // overwritten by the transposition)
             __syncthreads();
             if (threadIdx.x == 0) done_count = 0;
+            if (lane == 0) ent[dummy] = u32x4{kInvalidCorner, 0u, 0u, dummy};
             __syncthreads();
         }
     }

@@ -313,6 +313,7 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
         mxd::TileArgs t;
         rc = make_tile_args(d, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
         if (rc != MXD_OK) return rc;
+        t.store_vec = (hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
         e = mxd::launch_gradv_tiles(dtype, a, t, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: tile kernel launch failed: %s", hipGetErrorString(e));
     }

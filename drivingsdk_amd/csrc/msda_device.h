@@ -41,7 +41,7 @@ struct KArgs {
 
 // Launch description of the tile-ownership grad_value kernel.
 constexpr int kTilePx = 512;      // pixels per tile = threads per workgroup (a lane owns a pixel)
-constexpr int kTileEntCap = 512;  // list entries per wavefront and round
+constexpr int kTileEntCap = 448;  // list entries (16 bytes) per wavefront and round
 struct TileArgs {
     mxd_msda_plan map;     // only the XCD mapping fields are used: one "query" per work item
     int32_t tile_px;       // pixels per tile at most (<= kTilePx)
@@ -50,6 +50,7 @@ struct TileArgs {
     int32_t items_per_bh;  // upper bound of work items per (batch, head)
     int32_t vec;           // elements per load of a grad_out row
     int32_t accumulate;    // add into the existing contents of the image
+    int32_t store_vec;     // 4: rows of the image are 16-byte aligned, else 1
     uint32_t grid, block;
 };
 
