@@ -118,6 +118,12 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     const int lane = tid & (kWave - 1);
     const int wave = tid >> 6;
     const int npx = it.p1 - it.p0;
+    // A tile much smaller than the workgroup is held in several copies (lists and registers),
+    // each taking the samples of some queries; the copies meet in the image through atomics.
+    const int npx_pad = (npx + kLpp - 1) / kLpp * kLpp;
+    int copies = 1;
+    while (copies < 8 && 2 * copies * npx_pad <= kTilePx) copies *= 2;
+    const bool owned = it.exclusive && copies == 1;  // plain stores are enough
     const uint32_t seg = wave * kTileEntCap;  // this wavefront's entry storage
     uint32_t* cq = cq_all + wave * kCandCap;
 
@@ -225,6 +231,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     const float y = to_f32(__builtin_nontemporal_load(loc + 2 * e + 1));
                     const float aw = to_f32(__builtin_nontemporal_load(attn + e));
                     const Sample sm = sample_geometry(x, y, level, a.nk, true);
+                    const int copy_off = (q & (copies - 1)) * npx_pad;
 #pragma unroll
                     for (int r = 0; r < 2; ++r) {
                         const int pl = sm.pix[2 * r] - it.p0;  // left pixel of the pair, relative to the tile
@@ -232,12 +239,12 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                         const bool in_r = sm.cvalid[2 * r + 1] && pl + 1 >= 0 && pl + 1 < npx;
                         const bool pair = in_l && in_r && (pl % kLpp) != kLpp - 1;
                         if (in_l) {
-                            lst[2 * r] = pl;
+                            lst[2 * r] = pl + copy_off;
                             w0[2 * r] = sm.w[2 * r] * aw;
                             w1[2 * r] = pair ? sm.w[2 * r + 1] * aw : 0.0f;
                         }
                         if (in_r && !pair) {
-                            lst[2 * r + 1] = pl + 1;
+                            lst[2 * r + 1] = pl + 1 + copy_off;
                             w0[2 * r + 1] = sm.w[2 * r + 1] * aw;
                         }
                     }
@@ -336,7 +343,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
 
         // ---- write the CH channels of this tile -------------------------------------------
         const int nch = (hd - cb) < CH ? (hd - cb) : CH;
-        if (it.exclusive && t.store_vec == 4) {
+        if (owned && t.store_vec == 4) {
             // the lanes of a group hold a whole row of each of their pixels: 16-byte stores
             if (my_ch < hd) {
 #pragma unroll
@@ -376,11 +383,12 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 for (int k = 0; k < 32 * CH / kWave; ++k) {
                     const int idx = k * kWave + lane;
                     const int pl = idx / CH, c = idx % CH;
-                    const int px = px_base + pl;
-                    if (px < npx && c < nch) {
+                    const int vp = px_base + pl;             // pixel slot of the workgroup
+                    const int px = vp - (vp / npx_pad) * npx_pad;  // pixel of the tile (any copy)
+                    if (vp < copies * npx_pad && px < npx && c < nch) {
                         const float v = __builtin_bit_cast(float, (uint32_t)tr1[idx]);
                         float* dst = gimg + (int64_t)(it.p0 + px) * row_pitch + (int64_t)wk.h * hd + cb + c;
-                        if (!it.exclusive)
+                        if (!owned)
                             unsafeAtomicAdd(dst, v);
                         else if (t.accumulate)
                             *dst += v;
