@@ -18,6 +18,14 @@
 //     yields 0, the atomic is dropped by the hardware range check);
 //   * the geometry lanes turn the reduced dots into grad_attn / grad_loc and store them
 //     coalesced.
+//
+// SCATTER = false leaves grad_value to the tile-ownership pass (msda_bwd_tiles.hip) and hands it
+// the samples already sorted by tile: a sample is two "pair records" {pixel, query, weight of
+// that pixel, weight of the pixel to its right} (upper and lower corners).  The workgroup first
+// counts its records per tile in LDS (one geometry sweep over its sampling locations), turns
+// the counts into run starts inside its own slab of the record array, publishes them as its
+// row of the run table, and then -- where it computes grad_loc anyway -- drops every record
+// at the next free position of its tile's run (one LDS integer atomic per record).
 #include "msda_device.h"
 
 namespace mxd {
@@ -44,6 +52,64 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
+
+    // ---- records per tile of this workgroup: count, prefix, publish -----------------------
+    int32_t* tile_first = reinterpret_cast<int32_t*>(
+        smem + kMaxLevels * sizeof(i32x4) +
+        (size_t)a.plan.waves_per_block * a.plan.units_per_wave * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4)));
+    int32_t* cursor = tile_first + kMaxLevels;  // [tbl_stride] counts, then next free position per tile
+    u32x4* slab = nullptr;
+    if constexpr (!SCATTER) {
+        const int64_t wg_row = ((int64_t)wk.b * a.nh + wk.h) * a.nwg + wk.q_begin / a.plan.tile_q;
+        slab = a.rec + wg_row * a.rec_cap;
+        if (threadIdx.x == 0) {
+            int32_t first = 0;
+            for (int l = 0; l < a.nl; ++l) {
+                int32_t px;
+                tile_first[l] = first;
+                first += level_tile_count(lvl[l].x, lvl[l].y, lvl[l].z, a.nk, &px);
+            }
+        }
+        for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) cursor[i] = 0;
+        __syncthreads();
+        const T* loc0 = static_cast<const T*>(a.loc);
+        const int n = (wk.q_end - wk.q_begin) * a.S;
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const int qr = i / a.S, s = i - qr * a.S;
+            const int64_t e = (((int64_t)wk.b * a.nq + wk.q_begin + qr) * a.nh + wk.h) * a.S_full + s;
+            const int l = (int)(((uint32_t)s * a.np_magic) >> 20);
+            const Sample sm = sample_geometry(to_f32(loc0[2 * e]), to_f32(loc0[2 * e + 1]), lvl[l], a.nk, true);
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                if (sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) {
+                    const int32_t key = sm.cvalid[2 * r] ? sm.pix[2 * r] : sm.pix[2 * r + 1];
+                    atomicAdd(&cursor[tile_first[l] + ((key - lvl[l].z) >> kTilePxLog2)], 1);
+                }
+            }
+        }
+        __syncthreads();
+        if (wave == 0) {
+            // exclusive prefix over the counts, 64 at a time
+            int32_t carry = 0;
+            for (int base = 0; base < a.tbl_stride; base += kWave) {
+                const int i = base + lane;
+                const int32_t v = i < a.tbl_stride ? cursor[i] : 0;
+                int32_t inc = v;
+#pragma unroll
+                for (int d = 1; d < kWave; d <<= 1) {
+                    const int32_t o = __shfl_up(inc, d, kWave);
+                    if (lane >= d) inc += o;
+                }
+                if (i < a.tbl_stride) cursor[i] = carry + inc - v;
+                carry += __shfl(inc, kWave - 1, kWave);
+            }
+        }
+        __syncthreads();
+        uint32_t* row = a.tbl + wg_row * a.tbl_stride;
+        for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) row[i] = (uint32_t)cursor[i];
+        __syncthreads();  // the cursors are advanced from here on
+    }
+
     const int LPR = a.plan.lanes_per_row;
     const int lpr_log2 = __builtin_ctz(LPR);
     const int U = a.plan.units_per_wave;
@@ -205,10 +271,20 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     gloc[2 * e] = from_f32<T>(gx);
                     gloc[2 * e + 1] = from_f32<T>(gy);
                     if constexpr (!SCATTER) {
-                        // level-major key for the tile kernel: pixel index of the (y0, x0) corner
-                        const int p = s - l * a.np;
-                        a.keys[((((int64_t)wk.b * a.nh + wk.h) * a.nl + l) * a.nq + q) * a.np + p] =
-                            sm.valid ? sm.pix[0] : INT32_MIN;
+                        // pair records for the tile pass (same decisions as in the counting sweep)
+#pragma unroll
+                        for (int r = 0; r < 2; ++r) {
+                            const bool vl = sm.cvalid[2 * r], vr = sm.cvalid[2 * r + 1];
+                            if (vl || vr) {
+                                const int32_t key = vl ? sm.pix[2 * r] : sm.pix[2 * r + 1];
+                                const float wa = (vl ? sm.w[2 * r] : sm.w[2 * r + 1]) * aw;
+                                const float wb = (vl && vr) ? sm.w[2 * r + 1] * aw : 0.0f;
+                                const int32_t pos =
+                                    atomicAdd(&cursor[tile_first[l] + ((key - lvl[l].z) >> kTilePxLog2)], 1);
+                                slab[pos] = u32x4{(uint32_t)key, (uint32_t)q, __builtin_bit_cast(uint32_t, wa),
+                                                  __builtin_bit_cast(uint32_t, wb)};
+                            }
+                        }
                     }
                 }
             }

@@ -11,22 +11,22 @@
 // registers are fast, so the scatter is turned inside out:
 //
 //   * The pixels of every level are cut into tiles of kTilePx pixels.  A workgroup owns one
-//     tile of one (batch, head); every group of 4 lanes owns 4 pixels of the tile and keeps
+//     tile of one (batch, head); every group of 8 lanes owns 8 pixels of the tile and keeps
 //     their channels in registers for the whole kernel.
-//   * The backward's first kernel leaves, per sample, the pixel index of its top-left corner
-//     in a level-major key array.  The owner scans the keys of its (batch, head, level) --
-//     4 contiguous bytes per sample -- and rejects samples that cannot touch the tile with
-//     two compares.  Survivors are compacted (ballot + prefix) so that the geometry runs on
-//     dense batches of 64; per corner inside the tile an entry {query, weight} is appended to
-//     that PIXEL's linked list in LDS (one integer exchange on the list head; entry storage
-//     is private to the wavefront, so no allocation atomics are needed).
-//   * When the entry storage fills up (or the scan ends) the workgroup meets at a barrier and
-//     every lane group walks the lists of its own pixels: coalesced 16-byte loads of the
-//     grad_out row of the entry's query, fma into the registers.  No atomics, no
+//   * The backward's first kernel leaves its samples as pair records {pixel, query, weight,
+//     weight of the pixel to the right}, sorted by tile inside the slab of each of its
+//     workgroups, with a table of run starts.  The owner of a tile streams the runs of its
+//     tile (dense batches of 64 records, fetched one batch ahead) and appends an entry per
+//     record to the PIXEL's linked list in LDS (one integer exchange on the list head; entry
+//     storage is private to the wavefront, so no allocation atomics are needed).
+//   * When the entry storage fills up (or the input ends) the workgroup meets at a barrier and
+//     every lane group walks the lists of its own pixels: one coalesced load of the grad_out
+//     row of the entry's query per group, fma into the registers.  No atomics, no
 //     read-modify-write of shared accumulators.
-//   * At the end each wavefront passes its registers through LDS and writes whole rows:
-//     plain stores for tiles a single workgroup owns, a few atomics per workgroup for tiles of
-//     hot (coarse) levels, which are split over several workgroups by query range.
+//   * At the end plain 16-byte stores for tiles a single workgroup owns; tiles of hot (coarse)
+//     levels are split over several workgroups by query range and tiles much smaller than the
+//     workgroup are held in several copies: those pass their registers through LDS and add
+//     whole rows with a few atomics per workgroup.
 //
 // Which (level, tile, query chunk) a workgroup works on is derived on the device from
 // spatial_shapes / level_start_index, which never leave device memory; the host only needs
@@ -35,48 +35,56 @@
 
 namespace mxd {
 
-constexpr int kLpp = 8;                                  // lanes per pixel row = pixels per lane group
-constexpr int kScanBlocks = 4;                           // blocks of 64 keys fetched together
-constexpr int kCandCap = kWave + kScanBlocks * kWave;    // accepted candidates a wavefront can hold
+constexpr int kLpp = 8;  // lanes per pixel row = pixels per lane group
 
 // Work item table, evaluated identically by every workgroup.
 struct TileItem {
     int32_t level, H, W, base;   // level geometry
     int32_t p0, p1;              // pixel range of the tile, relative to the batch element
-    int32_t q0, q1;              // query range
+    int32_t w0, w1;              // range of workgroups of the first kernel whose records are taken
+    int32_t tile;                // index of the tile within the (batch, head): column of the run table
     int32_t exclusive;           // 1: no other workgroup touches this tile
 };
 
 __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32_t item, TileItem* out)
 {
-    int32_t first = 0;
+    // Items are numbered from the last level to the first: the coarse levels, whose tiles are
+    // split into many long-running items, start first and the short items of the fine levels
+    // fill the end of the launch.
+    int32_t tiles_after = 0;  // tiles of the levels not yet visited come first in the run table
     for (int l = 0; l < a.nl; ++l) {
+        int32_t P;
+        tiles_after += level_tile_count(a.shapes[2 * l], a.shapes[2 * l + 1], a.lsi[l], a.nk, &P);
+    }
+    int32_t first = 0;
+    for (int l = a.nl - 1; l >= 0; --l) {
         const int32_t H = a.shapes[2 * l], W = a.shapes[2 * l + 1], base = a.lsi[l];
-        if (H <= 0 || W <= 0) continue;
-        int64_t P = (int64_t)H * W;
-        if (base < 0 || base >= a.nk) continue;
-        if (base + P > a.nk) P = a.nk - base;  // never address past the value tensor
-        const int32_t nt = (int32_t)((P + t.tile_px - 1) / t.tile_px);
-        const int32_t tpx = (int32_t)((P + nt - 1) / nt);
-        const int64_t expect = ((int64_t)a.nq * a.np) / nt;
-        int32_t chunks = (int32_t)((expect + t.target - 1) / t.target);
+        int32_t P;
+        const int32_t nt = level_tile_count(H, W, base, a.nk, &P);
+        if (nt == 0) continue;
+        tiles_after -= nt;  // now the index of this level's first tile
+        // two pair records per sample, spread evenly over the tiles of the level
+        const int64_t expect = (2 * (int64_t)a.nq * a.np) / nt;
+        int64_t chunks = (expect + t.target - 1) / t.target;
         if (chunks < 1) chunks = 1;
         if (chunks > t.max_chunks) chunks = t.max_chunks;
-        const int32_t n = nt * chunks;
+        if (chunks > a.nwg) chunks = a.nwg;
+        const int32_t wpc = (int32_t)((a.nwg + chunks - 1) / chunks);  // first-kernel workgroups per chunk
+        chunks = (a.nwg + wpc - 1) / wpc;
+        const int32_t n = nt * (int32_t)chunks;
         if (item < first + n) {
-            const int32_t ti = (item - first) / chunks, ci = (item - first) % chunks;
-            const int32_t qc = (a.nq + chunks - 1) / chunks;
+            const int32_t ti = (item - first) / (int32_t)chunks, ci = (item - first) % (int32_t)chunks;
             out->level = l;
             out->H = H;
             out->W = W;
             out->base = base;
-            out->p0 = base + ti * tpx;
-            const int64_t e = (int64_t)out->p0 + tpx;
-            out->p1 = (int32_t)(e < base + P ? e : base + P);
-            out->q0 = ci * qc;
-            out->q1 = (out->q0 + qc) < a.nq ? (out->q0 + qc) : a.nq;
+            out->p0 = base + ti * kTilePx;
+            out->p1 = (out->p0 + kTilePx) < (base + P) ? (out->p0 + kTilePx) : (base + P);
+            out->w0 = ci * wpc;
+            out->w1 = (out->w0 + wpc) < a.nwg ? (out->w0 + wpc) : a.nwg;
+            out->tile = tiles_after + ti;
             out->exclusive = chunks == 1;
-            return out->p0 < out->p1 && out->q0 < out->q1;
+            return true;
         }
         first += n;
     }
@@ -84,7 +92,7 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
 }
 
 // CH = channels a lane group accumulates per pass (registers); heads with more channels are
-// done in several passes over the same candidates.  VEC = elements per load of a grad_out row.
+// done in several passes over the same records.  VEC = elements per load of a grad_out row.
 template <typename T, int CH, int VEC>
 __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArgs a, const TileArgs t)
 {
@@ -96,7 +104,9 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     // entry: {byte offset of the grad_out row, weight for the list's pixel, weight for the
     // next pixel, next entry of the same list}
     __shared__ u32x4 ent[NW * kTileEntCap];
-    __shared__ uint32_t cq_all[NW * kCandCap];          // accepted candidate indices, per wavefront
+    // up to 64 runs of records per wavefront at a time: first record, records before the run
+    __shared__ uint32_t run_src_all[NW * kWave];
+    __shared__ uint32_t run_pre_all[NW * kWave];
     __shared__ TileItem item_s;
     __shared__ int item_ok;
     __shared__ int done_count;
@@ -125,24 +135,15 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     while (copies < 8 && 2 * copies * npx_pad <= kTilePx) copies *= 2;
     const bool owned = it.exclusive && copies == 1;  // plain stores are enough
     const uint32_t seg = wave * kTileEntCap;  // this wavefront's entry storage
-    uint32_t* cq = cq_all + wave * kCandCap;
+    uint32_t* run_src = run_src_all + wave * kWave;
+    uint32_t* run_pre = run_pre_all + wave * kWave;
 
-    const T* loc = static_cast<const T*>(a.loc);
-    const T* attn = static_cast<const T*>(a.attn);
     const T* gout = static_cast<const T*>(a.grad_out);
-    const i32x4 level = {it.H, it.W, it.base, 0};
-    const int64_t bh_base = ((int64_t)wk.b * a.nq) * a.nh + wk.h;  // unit index = bh_base + q*nh
-    const int s_first = it.level * a.np;
-
-    // keys of this (batch, head, level), query-major then point: contiguous for a query range
-    const int32_t* keys = a.keys + ((((int64_t)wk.b * a.nh + wk.h) * a.nl + it.level) * a.nq) * a.np;
-    const int cand_begin = it.q0 * a.np, cand_end = it.q1 * a.np;
-    // contiguous share of the candidates per wavefront, in blocks of 64
-    const int nblk = (cand_end - cand_begin + kWave - 1) / kWave;
-    const int blk_per_wave = (nblk + NW - 1) / NW;
-    const int my_begin = cand_begin + wave * blk_per_wave * kWave;
-    int my_end = my_begin + blk_per_wave * kWave;
-    if (my_end > cand_end) my_end = cand_end;
+    const int64_t bh = (int64_t)wk.b * a.nh + wk.h;
+    const uint32_t* tbl = a.tbl + bh * a.nwg * a.tbl_stride + it.tile;
+    const u32x4* rec = a.rec + bh * a.nwg * a.rec_cap;
+    // runs of this wavefront: workgroups it.w0 + wave, + NW, + 2 NW, ... of the first kernel
+    const int nruns = (it.w1 - it.w0 - wave + NW - 1) / NW;  // <= 0: none
 
     float* gimg = a.grad_value + (size_t)wk.b * (a.gbatch_bytes / 4);
     const int64_t row_pitch = (int64_t)a.nh * hd;  // floats between neighbouring pixels
@@ -169,90 +170,93 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         // channels past head_dim re-read channel 0; their sums are never written out
         const int my_ch = cb + j * 4;
         const uint32_t lane_off = ghead_off + (uint32_t)(my_ch < hd ? my_ch : 0) * (uint32_t)sizeof(T);
+        const int nch = (hd - cb) < CH ? (hd - cb) : CH;
 
-        int cursor = my_begin;   // next unscanned candidate of this wavefront (uniform)
-        int32_t pre[kScanBlocks];  // keys of the blocks at `cursor`, fetched one step ahead
-        auto load_keys = [&](int base) {
+        // input state of this wavefront (uniform): next group of runs, records of the current
+        // group, next unread record, and the batch fetched ahead
+        int rg = 0, N = 0, i0 = 0;
+        u32x4 ahead = {0u, 0u, 0u, 0u};
+        auto fetch_ahead = [&](int first) {
+            const int i = first + lane;
+            if (i < N) {
+                int r = 0;
 #pragma unroll
-            for (int jb = 0; jb < kScanBlocks; ++jb) {
-                const int idx = base + jb * kWave + lane;
-                pre[jb] = idx < my_end ? __builtin_nontemporal_load(keys + idx) : INT32_MIN;
+                for (int step = kWave / 2; step > 0; step >>= 1)
+                    if (run_pre[r + step] <= (uint32_t)i) r += step;
+                ahead = __builtin_nontemporal_load(rec + (run_src[r] + ((uint32_t)i - run_pre[r])));
             }
         };
-        load_keys(my_begin);
-        int ncq = 0;             // accepted candidates waiting in cq (uniform)
         bool counted = false;    // this wavefront has reported the end of its work
         while (true) {
-            // ---- scan keys, compact accepted candidates, append list entries ---------------
+            // ---- stream records, append list entries ------------------------------------------
             int count = 0;  // entries of this wavefront in this round (uniform)
+            fetch_ahead(i0);  // (again after a walk: the batch fetched ahead is not kept across it)
             while (true) {
-                // (1) refill the candidate queue from the keys fetched one step ahead, and put the
-                // next kScanBlocks blocks of 64 keys in flight before testing the current ones
-                while (cursor < my_end && ncq < kWave) {
-                    int32_t key[kScanBlocks];
+                if (i0 >= N) {
+                    if (rg >= nruns) break;  // input exhausted
+                    // next group of up to 64 runs: one run per lane
+                    const int r = rg + lane;
+                    uint32_t len = 0, src = 0;
+                    if (r < nruns) {
+                        const int w = it.w0 + wave + NW * r;
+                        const uint32_t* row = tbl + (size_t)w * a.tbl_stride;
+                        const uint32_t s = row[0];
+                        len = row[1] - s;
+                        src = (uint32_t)w * (uint32_t)a.rec_cap + s;
+                    }
+                    uint32_t inc = len;
 #pragma unroll
-                    for (int jb = 0; jb < kScanBlocks; ++jb) key[jb] = pre[jb];
-                    load_keys(cursor + kScanBlocks * kWave);
-#pragma unroll
-                    for (int jb = 0; jb < kScanBlocks; ++jb) {
-                        // corners are key, key+1, key+W, key+W+1
-                        const bool maybe =
-                            (key[jb] != INT32_MIN) && ((int64_t)key[jb] + it.W + 1 >= it.p0) && (key[jb] < it.p1);
-                        const uint64_t mask = __ballot(maybe);
-                        if (mask) {
-                            if (maybe)
-                                cq[ncq + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
-                                                                   __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0))] =
-                                    cursor + jb * kWave + lane;
-                            ncq += __builtin_popcountll(mask);
+                    for (int d = 1; d < kWave; d <<= 1) {
+                        const uint32_t o = __shfl_up(inc, d, kWave);
+                        if (lane >= d) inc += o;
+                    }
+                    wave_lds_sync();
+                    run_src[lane] = src;
+                    run_pre[lane] = inc - len;
+                    wave_lds_sync();
+                    N = (int)__shfl(inc, kWave - 1, kWave);
+                    rg += kWave;
+                    i0 = 0;
+                    fetch_ahead(0);
+                    continue;
+                }
+                if (count + 2 * kWave > (int)kDummyOfWave) break;  // entry storage full: next round
+                const bool have = i0 + lane < N;
+                const u32x4 rc = ahead;
+                i0 += kWave;
+                fetch_ahead(i0);
+                // A record is the pair (pixel, pixel + 1).  A pair whose pixels belong to the same
+                // lane group becomes ONE entry in the list of the left pixel (the grad_out row is
+                // fetched once for both); otherwise each pixel gets an entry of its own.  The right
+                // pixel of the last pixel of the tile belongs to the next tile: added with atomics.
+                int lst[2] = {-1, -1};
+                float w0[2] = {0.f, 0.f}, w1[2] = {0.f, 0.f};
+                uint32_t q = 0;
+                bool spill = false;
+                float wb = 0.f;
+                if (have) {
+                    const uint32_t kx = rc.x, qx = rc.y, ya = rc.z, za = rc.w;
+                    q = qx;
+                    const int pl = (int)kx - it.p0;
+                    const float wa = __builtin_bit_cast(float, ya);
+                    wb = __builtin_bit_cast(float, za);
+                    const int copy_off = (int)(q & (uint32_t)(copies - 1)) * npx_pad;
+                    const bool in_r = pl + 1 < npx;
+                    const bool pair = in_r && (pl % kLpp) != kLpp - 1;
+                    lst[0] = pl + copy_off;
+                    w0[0] = wa;
+                    w1[0] = pair ? wb : 0.0f;
+                    if (!pair && wb != 0.0f) {
+                        if (in_r) {
+                            lst[1] = pl + 1 + copy_off;
+                            w0[1] = wb;
+                        } else {
+                            spill = true;
                         }
                     }
-                    cursor += kScanBlocks * kWave;
                 }
-                // (2) a dense batch of accepted candidates: geometry + list append
-                const bool flush_tail = cursor >= my_end && ncq > 0;
-                if (!(ncq >= kWave || flush_tail)) break;                      // nothing left to do
-                if (count + 4 * kWave > (int)kDummyOfWave) break;              // entry storage full: next round
-                const int take = ncq < kWave ? ncq : kWave;
-                wave_lds_sync();
-                // A sample touches two pixel pairs (p, p+1): its upper and its lower corners.  A pair
-                // whose pixels belong to the same lane group becomes ONE entry in the list of the left
-                // pixel (the grad_out row is fetched once for both); otherwise each corner inside the
-                // tile gets an entry of its own with no weight for the neighbour.
-                int lst[4] = {-1, -1, -1, -1};   // list (pixel inside the tile) of up to 4 entries
-                float w0[4] = {0.f, 0.f, 0.f, 0.f}, w1[4] = {0.f, 0.f, 0.f, 0.f};
-                int q = 0;
-                if (lane < take) {
-                    const int idx = cq[ncq - take + lane];
-                    q = idx / a.np;
-                    const int p = idx - q * a.np;
-                    const int64_t e = (bh_base + (int64_t)q * a.nh) * a.S_full + s_first + p;
-                    const float x = to_f32(__builtin_nontemporal_load(loc + 2 * e));
-                    const float y = to_f32(__builtin_nontemporal_load(loc + 2 * e + 1));
-                    const float aw = to_f32(__builtin_nontemporal_load(attn + e));
-                    const Sample sm = sample_geometry(x, y, level, a.nk, true);
-                    const int copy_off = (q & (copies - 1)) * npx_pad;
 #pragma unroll
-                    for (int r = 0; r < 2; ++r) {
-                        const int pl = sm.pix[2 * r] - it.p0;  // left pixel of the pair, relative to the tile
-                        const bool in_l = sm.cvalid[2 * r] && pl >= 0 && pl < npx;
-                        const bool in_r = sm.cvalid[2 * r + 1] && pl + 1 >= 0 && pl + 1 < npx;
-                        const bool pair = in_l && in_r && (pl % kLpp) != kLpp - 1;
-                        if (in_l) {
-                            lst[2 * r] = pl + copy_off;
-                            w0[2 * r] = sm.w[2 * r] * aw;
-                            w1[2 * r] = pair ? sm.w[2 * r + 1] * aw : 0.0f;
-                        }
-                        if (in_r && !pair) {
-                            lst[2 * r + 1] = pl + 1 + copy_off;
-                            w0[2 * r + 1] = sm.w[2 * r + 1] * aw;
-                        }
-                    }
-                }
-                ncq -= take;
-                wave_lds_sync();
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
+                for (int k = 0; k < 2; ++k) {
                     const bool push = lst[k] >= 0;
                     const uint64_t mask = __ballot(push);
                     if (mask) {
@@ -261,14 +265,26 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                                                  __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                                                            __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
                             const uint32_t next = atomicExch(&heads[lst[k]], pos);
-                            ent[pos] = u32x4{(uint32_t)q * row_bytes, __builtin_bit_cast(uint32_t, w0[k]),
+                            ent[pos] = u32x4{q * row_bytes, __builtin_bit_cast(uint32_t, w0[k]),
                                              __builtin_bit_cast(uint32_t, w1[k]), next};
                         }
                         count += __builtin_popcountll(mask);
                     }
                 }
+                // pairs that reach into the next tile: one at a time, the wavefront adds the row
+                uint64_t smask = __ballot(spill);
+                while (smask) {
+                    const int src_lane = __builtin_ctzll(smask);
+                    smask &= smask - 1;
+                    const uint32_t sq = __builtin_amdgcn_readlane(q, src_lane);
+                    const float sw = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(uint32_t, wb), src_lane));
+                    if (lane < nch) {
+                        const float g = to_f32(gout[((int64_t)wk.b * a.nq + sq) * row_pitch + (int64_t)wk.h * hd + cb + lane]);
+                        unsafeAtomicAdd(gimg + (int64_t)it.p1 * row_pitch + (int64_t)wk.h * hd + cb + lane, sw * g);
+                    }
+                }
             }
-            if (cursor >= my_end && ncq == 0 && !counted) {
+            if (rg >= nruns && i0 >= N && !counted) {
                 counted = true;
                 if (lane == 0) atomicAdd(&done_count, 1);
             }
@@ -279,8 +295,8 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
             // The lanes of a group read one grad_out row with ONE coalesced load (lane j: channels
             // 4j..4j+3): the memory pipeline's cost is per cache line touched by an instruction.
             // The loop body is branch-free: a list that has ended keeps "reading" the dummy entry.
-            // Two lists are walked together, two entries of each per trip, so that four row loads
-            // are in flight while the fmas of the previous ones run.
+            // Four lists are walked together, one entry of each per trip: four independent row
+            // loads in flight, no loop-carried row data (other wavefronts cover the load latency).
             {
                 auto fetch = [&](uint32_t& e, float (&g)[CHL], float& wa, float& wb) {
                     const u32x4 en = ent[e];
@@ -298,43 +314,29 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     e = en.w;
                 };
 #pragma unroll
-                for (int i = 0; i < kLpp; i += 2) {
+                for (int i = 0; i < kLpp; i += 4) {
                     const int px = grp * kLpp + i;
-                    uint32_t ea = heads[px], eb = heads[px + 1];
+                    uint32_t e[4];
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) e[m] = heads[px + m];
                     if (j == 0) {  // same wavefront: ordered after the reads above
-                        heads[px] = dummy;
-                        heads[px + 1] = dummy;
-                    }
-                    float ga0[CHL], ga1[CHL], gb0[CHL], gb1[CHL];
-                    float ua0, va0, ua1, va1, ub0, vb0, ub1, vb1;
-                    auto fma_a = [&](const float (&g)[CHL], float u, float v) {
 #pragma unroll
-                        for (int c = 0; c < CHL; ++c) {
-                            acc[i][c] = __builtin_fmaf(u, g[c], acc[i][c]);
-                            acc[i + 1][c] = __builtin_fmaf(v, g[c], acc[i + 1][c]);
-                        }
-                    };
-                    auto fma_b = [&](const float (&g)[CHL], float u, float v) {
-#pragma unroll
-                        for (int c = 0; c < CHL; ++c) {
-                            acc[i + 1][c] = __builtin_fmaf(u, g[c], acc[i + 1][c]);
-                            if (i + 2 < kLpp) acc[(i + 2) % kLpp][c] = __builtin_fmaf(v, g[c], acc[(i + 2) % kLpp][c]);
-                        }
-                    };
-                    fetch(ea, ga0, ua0, va0);
-                    fetch(eb, gb0, ub0, vb0);
-                    while (__ballot(ea != dummy || eb != dummy)) {
-                        fetch(ea, ga1, ua1, va1);
-                        fetch(eb, gb1, ub1, vb1);
-                        fma_a(ga0, ua0, va0);
-                        fma_b(gb0, ub0, vb0);
-                        fetch(ea, ga0, ua0, va0);
-                        fetch(eb, gb0, ub0, vb0);
-                        fma_a(ga1, ua1, va1);
-                        fma_b(gb1, ub1, vb1);
+                        for (int m = 0; m < 4; ++m) heads[px + m] = dummy;
                     }
-                    fma_a(ga0, ua0, va0);
-                    fma_b(gb0, ub0, vb0);
+                    while (__ballot((e[0] != dummy) | (e[1] != dummy) | (e[2] != dummy) | (e[3] != dummy))) {
+                        float g[4][CHL], u[4], v[4];
+#pragma unroll
+                        for (int m = 0; m < 4; ++m) fetch(e[m], g[m], u[m], v[m]);
+#pragma unroll
+                        for (int m = 0; m < 4; ++m) {
+#pragma unroll
+                            for (int c = 0; c < CHL; ++c) {
+                                acc[i + m][c] = __builtin_fmaf(u[m], g[m][c], acc[i + m][c]);
+                                if (i + m + 1 < kLpp)
+                                    acc[(i + m + 1) % kLpp][c] = __builtin_fmaf(v[m], g[m][c], acc[(i + m + 1) % kLpp][c]);
+                            }
+                        }
+                    }
                 }
             }
             __syncthreads();
@@ -342,19 +344,30 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         }
 
         // ---- write the CH channels of this tile -------------------------------------------
-        const int nch = (hd - cb) < CH ? (hd - cb) : CH;
+        // (address arithmetic derived from these opaque copies stays inside this section instead of
+        // occupying registers during the rounds)
+        int grp_w = grp, lane_w = lane;
+        asm volatile("" : "+v"(grp_w), "+v"(lane_w));
         if (owned && t.store_vec == 4) {
             // the lanes of a group hold a whole row of each of their pixels: 16-byte stores
             if (my_ch < hd) {
 #pragma unroll
                 for (int i = 0; i < kLpp; ++i) {
-                    const int px = grp * kLpp + i;
+                    const int px = grp_w * kLpp + i;
                     if (px < npx) {
                         f32x4* dst = reinterpret_cast<f32x4*>(gimg + (int64_t)(it.p0 + px) * row_pitch +
                                                               (int64_t)wk.h * hd + my_ch);
                         f32x4 v = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
-                        if (t.accumulate) v += *dst;
-                        *dst = v;
+                        if (px == 0) {
+                            // the first pixel of a tile also receives, through atomics, the right
+                            // halves of pairs that start on the last pixel of the previous tile
+                            float* d1 = reinterpret_cast<float*>(dst);
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) unsafeAtomicAdd(d1 + c, v[c]);
+                        } else {
+                            if (t.accumulate) v += *dst;
+                            *dst = v;
+                        }
                     }
                 }
             }
@@ -369,8 +382,8 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
             const u32_alias* tr1 = reinterpret_cast<const u32_alias*>(tr4);
             for (int half = 0; half < 2; ++half) {
                 wave_lds_sync();
-                if (((lane / kLpp) >> 2) == half) {
-                    const int gl = (lane / kLpp) & 3;
+                if (((lane_w / kLpp) >> 2) == half) {
+                    const int gl = (lane_w / kLpp) & 3;
 #pragma unroll
                     for (int i = 0; i < kLpp; ++i)
                         tr4[(gl * kLpp + i) * (CH / 4) + j] =
@@ -381,14 +394,14 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 const int px_base = wave * kWave + half * 32;
 #pragma unroll 4
                 for (int k = 0; k < 32 * CH / kWave; ++k) {
-                    const int idx = k * kWave + lane;
+                    const int idx = k * kWave + lane_w;
                     const int pl = idx / CH, c = idx % CH;
                     const int vp = px_base + pl;             // pixel slot of the workgroup
                     const int px = vp - (vp / npx_pad) * npx_pad;  // pixel of the tile (any copy)
                     if (vp < copies * npx_pad && px < npx && c < nch) {
                         const float v = __builtin_bit_cast(float, (uint32_t)tr1[idx]);
                         float* dst = gimg + (int64_t)(it.p0 + px) * row_pitch + (int64_t)wk.h * hd + cb + c;
-                        if (!owned)
+                        if (!owned || px == 0)
                             unsafeAtomicAdd(dst, v);
                         else if (t.accumulate)
                             *dst += v;

@@ -98,23 +98,53 @@ int64_t fill_xcd_map(mxd_msda_plan* p, int64_t bs, int64_t nh, int64_t ntiles)
     return bs * nh * ntiles;
 }
 
+// How the backward pass is laid out for a problem size: whether grad_value goes through the
+// tile-ownership pass (and then the hand-over buffers between its two kernels) or through
+// global atomics, and where things live in the caller's workspace.
+//   workspace = [run table][pair records][fp32 image of grad_value, 16-bit dtypes only]
+constexpr int64_t kBwdTileQ = 256;  // queries per workgroup of the first kernel (tile pass)
+struct BwdLayout {
+    bool tiles;          // false: one kernel with global atomics
+    int64_t nwg;         // workgroups of the first kernel per (batch, head)
+    int64_t rec_cap;     // pair records per workgroup slab: 2 per sample
+    int64_t tbl_stride;  // tiles per (batch, head) at most, plus one
+    size_t tbl_bytes, rec_bytes, image_bytes, total;
+};
+
+BwdLayout bwd_layout(int dtype, const Dims& d)
+{
+    BwdLayout L;
+    memset(&L, 0, sizeof(L));
+    L.nwg = (d.nq + kBwdTileQ - 1) / kBwdTileQ;
+    L.rec_cap = 2 * kBwdTileQ * d.nl * d.np;
+    // a level has at most nk/kTilePx + 1 tiles whatever spatial_shapes says
+    L.tbl_stride = d.nl * (d.nk / mxd::kTilePx + 1) + 1;
+    const int64_t tbl = d.bs * d.nh * L.nwg * L.tbl_stride * 4;
+    L.tiles = env_int("MXD_MSDA_BWD_ATOMIC", 0) == 0 &&
+              L.tbl_stride <= 4096 &&                      // counters of the first kernel live in LDS
+              tbl <= (int64_t(1) << 28) &&                 // run table of at most 256 MiB
+              L.nwg * L.rec_cap < (int64_t(1) << 31) &&    // 32-bit record indices within a (batch, head)
+              d.nq * d.nh * d.hd * 4 < (int64_t(1) << 31); // grad_output rows addressed with 32-bit byte offsets
+    if (L.tiles) {
+        L.tbl_bytes = ((size_t)tbl + 255) & ~(size_t)255;
+        L.rec_bytes = (size_t)d.bs * d.nh * L.nwg * L.rec_cap * 16;
+    }
+    if (elem_size(dtype) == 2) L.image_bytes = (size_t)d.bs * d.nk * d.nh * d.hd * 4;
+    L.total = L.tbl_bytes + L.rec_bytes + L.image_bytes;
+    return L;
+}
+
 // Geometry of the tile-ownership grad_value kernel (msda_bwd_tiles.hip).
-int make_tile_args(const Dims& d, int vec, int accumulate, mxd::TileArgs* t)
+int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, mxd::TileArgs* t)
 {
     memset(t, 0, sizeof(*t));
-    int64_t tile_px = mxd::kTilePx;
-    if (tile_px > d.nk) tile_px = d.nk;
-    t->tile_px = (int32_t)tile_px;
-    t->target = env_int("MXD_MSDA_TILE_TARGET", 4096);
-    if (t->target < 64) t->target = 64;
+    t->target = env_int("MXD_MSDA_TILE_TARGET", 8192);
+    if (t->target < 128) t->target = 128;
     t->max_chunks = 64;
-    // work items per (batch, head): sum over levels of tiles*chunks <= nl*nq*np/target + sum of tiles,
-    // and a level has at most nk/tile_px + 1 tiles whatever spatial_shapes says
-    const int64_t items = (d.nl * d.nq * d.np + t->target - 1) / t->target + d.nl * (d.nk / tile_px + 1);
+    // work items per (batch, head): sum over levels of tiles*chunks <= 2*nl*nq*np/target + nl + sum of tiles
+    const int64_t items = d.nl * ((2 * d.nq * d.np + t->target - 1) / t->target + 1) + L.tbl_stride;
     if (items >= (int64_t(1) << 24)) return fail(MXD_E_SHAPE, "backward needs %lld work items per (batch, head)", (long long)items);
     t->items_per_bh = (int32_t)items;
-    if (d.nq * d.nh * d.hd * 4 >= (int64_t(1) << 31))
-        return fail(MXD_E_SHAPE, "one batch element of grad_output (num_queries*num_heads*embed_dims) must stay below 2 GiB at 4 bytes per element");
     t->vec = vec;
     t->accumulate = accumulate;
     t->map.tile_q = 1;
@@ -144,8 +174,11 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     p->npass = npass;
     p->units_per_wave = mxd::kWave / lpr;
     p->waves_per_block = 4;
-    int iters = env_int(backward ? "MXD_MSDA_BWD_ITERS" : "MXD_MSDA_FWD_ITERS", 1);
+    int iters = env_int("MXD_MSDA_FWD_ITERS", 1);
     if (iters < 1) iters = 1;
+    const BwdLayout L = bwd_layout(dtype, d);
+    // the tile pass wants kBwdTileQ queries per workgroup of the first backward kernel
+    if (backward) iters = L.tiles ? (int)(kBwdTileQ / (p->units_per_wave * p->waves_per_block)) : 1;
     p->iters = iters;
     p->tile_q = p->units_per_wave * p->waves_per_block * p->iters;
     const int64_t ntiles = (d.nq + p->tile_q - 1) / p->tile_q;
@@ -157,6 +190,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     size_t per_unit = mxd::kChunkStride * sizeof(mxd::Entry);
     if (backward) per_unit += mxd::kChunk * sizeof(mxd::f32x4);
     p->lds_bytes = (uint32_t)(mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)p->waves_per_block * p->units_per_wave * per_unit);
+    if (backward && L.tiles) p->lds_bytes += (uint32_t)((mxd::kMaxLevels + L.tbl_stride) * sizeof(int32_t));
     return MXD_OK;
 }
 
@@ -242,21 +276,12 @@ int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int
     return MXD_OK;
 }
 
-// workspace layout: [keys: bs*nh*nl*nq*np int32, padded to 256 B][fp32 image of grad_value, 16-bit dtypes only]
-static size_t keys_bytes(const Dims& d)
-{
-    const size_t n = (size_t)d.bs * d.nh * d.nl * d.nq * d.np * 4;
-    return (n + 255) & ~(size_t)255;
-}
-
 size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
                                          int64_t nl_attn, int64_t nq, int64_t np)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     if (check_dims(dtype, d) != MXD_OK) return 0;
-    size_t n = keys_bytes(d);
-    if (elem_size(dtype) == 2) n += (size_t)bs * nk * nh * hd * 4;
-    return n;
+    return bwd_layout(dtype, d).total;
 }
 
 int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
@@ -271,18 +296,18 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !grad_output || !grad_value ||
         !grad_loc || !grad_attn)
         return fail(MXD_E_NULL, "mxd_msda_backward: NULL data pointer");
-    const size_t need = mxd_msda_backward_workspace_bytes(dtype, bs, nk, nh, hd, nl, nl_attn, nq, np);
-    if (!workspace || workspace_bytes < need)
+    const BwdLayout L = bwd_layout(dtype, d);
+    const size_t need = L.total;
+    if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace of %zu bytes required, %zu given", need,
                     workspace ? workspace_bytes : (size_t)0);
-    if (reinterpret_cast<uintptr_t>(workspace) & 15u)
+    if (need > 0 && (reinterpret_cast<uintptr_t>(workspace) & 15u))
         return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace must be 16-byte aligned");
     const bool half = elem_size(dtype) == 2;
     if ((flags & MXD_BWD_ACCUMULATE) && half)
         return fail(MXD_E_DTYPE, "mxd_msda_backward: MXD_BWD_ACCUMULATE is only available for float32");
-    int32_t* keys = static_cast<int32_t*>(workspace);
-    float* image = half ? reinterpret_cast<float*>(static_cast<char*>(workspace) + keys_bytes(d))
-                        : static_cast<float*>(grad_value);
+    char* ws = static_cast<char*>(workspace);
+    float* image = half ? reinterpret_cast<float*>(ws + L.tbl_bytes + L.rec_bytes) : static_cast<float*>(grad_value);
     if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_msda_backward: grad_value is not 4-byte aligned");
     int align = ptr_align(value);
     if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
@@ -298,7 +323,11 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     a.attn = attn_weight;
     a.grad_out = grad_output;
     a.grad_value = image;
-    a.keys = keys;
+    a.tbl = reinterpret_cast<uint32_t*>(ws);
+    a.rec = reinterpret_cast<mxd::u32x4*>(ws + L.tbl_bytes);
+    a.nwg = (int32_t)L.nwg;
+    a.rec_cap = (int32_t)L.rec_cap;
+    a.tbl_stride = (int32_t)L.tbl_stride;
     a.grad_loc = grad_loc;
     a.grad_attn = grad_attn;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
@@ -306,12 +335,12 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     hipError_t e = hipSuccess;
     if (!(flags & MXD_BWD_ACCUMULATE)) e = mxd::launch_fill_zero(image, n, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: zero-fill launch failed: %s", hipGetErrorString(e));
-    const bool atomic_mode = env_int("MXD_MSDA_BWD_ATOMIC", 0) != 0;
+    const bool atomic_mode = !L.tiles;
     e = mxd::launch_backward(dtype, a, atomic_mode, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: launch failed: %s", hipGetErrorString(e));
     if (!atomic_mode) {
         mxd::TileArgs t;
-        rc = make_tile_args(d, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
+        rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
         if (rc != MXD_OK) return rc;
         t.store_vec = (hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
         e = mxd::launch_gradv_tiles(dtype, a, t, stream);

@@ -28,7 +28,16 @@ struct KArgs {
     float* grad_value;     // fp32 accumulation image of grad_value
     void* grad_loc;
     void* grad_attn;
-    int32_t* keys;         // [bs, nh, nl, nq, np] pixel index of each sample's top-left corner (INT32_MIN: invalid)
+    // Hand-over from the first backward kernel to the grad_value pass.  Every workgroup of the
+    // first kernel (tile_q queries of one (batch, head)) owns a slab of rec_cap pair records,
+    // which it fills sorted by tile; row [w] of the table holds the start of every tile's run
+    // inside slab w (tbl_stride entries, the last used one being the total).
+    // record = {pixel index, query, weight of that pixel, weight of the pixel to its right}
+    u32x4* rec;            // [bs*nh][nwg][rec_cap]
+    uint32_t* tbl;         // [bs*nh][nwg][tbl_stride]
+    int32_t nwg;           // workgroups of the first kernel per (batch, head)
+    int32_t rec_cap;       // 2 * tile_q * nl * np
+    int32_t tbl_stride;    // upper bound of tiles per (batch, head), plus one
     int32_t bs, nk, nh, hd, nl, np, nq;
     int32_t S;             // nl*np: samples per unit that are evaluated
     int32_t S_full;        // nl_attn*np: samples per unit that are stored
@@ -40,12 +49,10 @@ struct KArgs {
 };
 
 // Launch description of the tile-ownership grad_value kernel.
-constexpr int kTilePx = 512;      // pixels per tile = threads per workgroup (a lane owns a pixel)
-constexpr int kTileEntCap = 448;  // list entries (16 bytes) per wavefront and round
+constexpr int kTileEntCap = 576;  // list entries (16 bytes) per wavefront and round
 struct TileArgs {
     mxd_msda_plan map;     // only the XCD mapping fields are used: one "query" per work item
-    int32_t tile_px;       // pixels per tile at most (<= kTilePx)
-    int32_t target;        // samples per work item aimed at when a hot tile is split by query range
+    int32_t target;        // pair records per work item aimed at when a hot tile is split by query range
     int32_t max_chunks;    // most query chunks a tile is split into
     int32_t items_per_bh;  // upper bound of work items per (batch, head)
     int32_t vec;           // elements per load of a grad_out row

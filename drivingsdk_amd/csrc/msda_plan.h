@@ -29,9 +29,24 @@ constexpr int kMaxLevels = 64;
 constexpr int kChunk = 16;           // samples of a unit staged per pass
 constexpr int kChunkStride = 17;     // staged entries per unit incl. one pad entry (LDS banks)
 
+constexpr int kTilePx = 512;         // pixels per tile of the grad_value pass = threads of its workgroups
+constexpr int kTilePxLog2 = 9;
+
 struct Work {
     int32_t b, h, q_begin, q_end;
 };
+
+// Tiles of the grad_value pass that a level contributes: its pixels [base, base + H*W), clipped
+// to the value tensor, in pieces of kTilePx.  *pixels receives the clipped pixel count.
+MXD_HD inline int32_t level_tile_count(int32_t H, int32_t W, int32_t base, int32_t nk, int32_t* pixels)
+{
+    *pixels = 0;
+    if (H <= 0 || W <= 0 || base < 0 || base >= nk) return 0;
+    int64_t P = (int64_t)H * W;
+    if (base + P > nk) P = nk - base;  // never address past the value tensor
+    *pixels = (int32_t)P;
+    return (int32_t)((P + kTilePx - 1) >> kTilePxLog2);
+}
 
 // Decode a workgroup index.  Returns false when the workgroup has nothing to do.
 MXD_HD inline bool decode_block(const mxd_msda_plan& p, uint32_t bid, int32_t bs, int32_t nh, int32_t nq, Work* w)
