@@ -281,8 +281,8 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                                 const float wb = (vl && vr) ? sm.w[2 * r + 1] * aw : 0.0f;
                                 const int32_t pos =
                                     atomicAdd(&cursor[tile_first[l] + ((key - lvl[l].z) >> kTilePxLog2)], 1);
-                                slab[pos] = u32x4{(uint32_t)key, (uint32_t)q, __builtin_bit_cast(uint32_t, wa),
-                                                  __builtin_bit_cast(uint32_t, wb)};
+                                __builtin_nontemporal_store(u32x4{(uint32_t)key, (uint32_t)q, __builtin_bit_cast(uint32_t, wa),
+                                                                  __builtin_bit_cast(uint32_t, wb)}, slab + pos);
                             }
                         }
                     }

@@ -102,9 +102,15 @@ int64_t fill_xcd_map(mxd_msda_plan* p, int64_t bs, int64_t nh, int64_t ntiles)
 // tile-ownership pass (and then the hand-over buffers between its two kernels) or through
 // global atomics, and where things live in the caller's workspace.
 //   workspace = [run table][pair records][fp32 image of grad_value, 16-bit dtypes only]
-constexpr int64_t kBwdTileQ = 256;  // queries per workgroup of the first kernel (tile pass)
+// queries per workgroup of the first kernel (tile pass): 64, 128 or 256
+static int64_t bwd_tile_q()
+{
+    const int v = env_int("MXD_MSDA_BWD_TILE_Q", 128);
+    return v == 64 || v == 256 ? v : 128;
+}
 struct BwdLayout {
     bool tiles;          // false: one kernel with global atomics
+    int64_t tile_q;      // queries per workgroup of the first kernel
     int64_t nwg;         // workgroups of the first kernel per (batch, head)
     int64_t rec_cap;     // pair records per workgroup slab: 2 per sample
     int64_t tbl_stride;  // tiles per (batch, head) at most, plus one
@@ -115,8 +121,9 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
 {
     BwdLayout L;
     memset(&L, 0, sizeof(L));
-    L.nwg = (d.nq + kBwdTileQ - 1) / kBwdTileQ;
-    L.rec_cap = 2 * kBwdTileQ * d.nl * d.np;
+    L.tile_q = bwd_tile_q();
+    L.nwg = (d.nq + L.tile_q - 1) / L.tile_q;
+    L.rec_cap = 2 * L.tile_q * d.nl * d.np;
     // a level has at most nk/kTilePx + 1 tiles whatever spatial_shapes says
     L.tbl_stride = d.nl * (d.nk / mxd::kTilePx + 1) + 1;
     const int64_t tbl = d.bs * d.nh * L.nwg * L.tbl_stride * 4;
@@ -138,7 +145,13 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
 int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, mxd::TileArgs* t)
 {
     memset(t, 0, sizeof(*t));
-    t->target = env_int("MXD_MSDA_TILE_TARGET", 8192);
+    // pair records per work item when a hot tile is split: enough items to fill the 512 workgroup
+    // slots of the chip about twice (measured optimum on MI355X; fewer, longer items lose to imbalance,
+    // more, shorter ones to the atomics of their write-out)
+    int64_t target = 2 * d.bs * d.nh * d.nq * d.nl * d.np / 640;
+    if (target < 8192) target = 8192;
+    if (target > 32768) target = 32768;
+    t->target = env_int("MXD_MSDA_TILE_TARGET", (int)target);
     if (t->target < 128) t->target = 128;
     t->max_chunks = 64;
     // work items per (batch, head): sum over levels of tiles*chunks <= 2*nl*nq*np/target + nl + sum of tiles
@@ -177,8 +190,8 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     int iters = env_int("MXD_MSDA_FWD_ITERS", 1);
     if (iters < 1) iters = 1;
     const BwdLayout L = bwd_layout(dtype, d);
-    // the tile pass wants kBwdTileQ queries per workgroup of the first backward kernel
-    if (backward) iters = L.tiles ? (int)(kBwdTileQ / (p->units_per_wave * p->waves_per_block)) : 1;
+    // the tile pass wants L.tile_q queries per workgroup of the first backward kernel
+    if (backward) iters = L.tiles ? (int)(L.tile_q / (p->units_per_wave * p->waves_per_block)) : 1;
     p->iters = iters;
     p->tile_q = p->units_per_wave * p->waves_per_block * p->iters;
     const int64_t ntiles = (d.nq + p->tile_q - 1) / p->tile_q;
