@@ -113,6 +113,13 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
 
     Work wk;
     if (!decode_block(t.map, blockIdx.x, a.bs, a.nh, t.items_per_bh, &wk)) return;
+    {
+        // item-major, batch-minor: the long-running items (coarse levels, numbered first) of every
+        // batch element start at the beginning of the launch
+        const int64_t r = (int64_t)wk.b * t.items_per_bh + wk.q_begin;
+        wk.b = (int32_t)(r % a.bs);
+        wk.q_begin = (int32_t)(r / a.bs);
+    }
     if (threadIdx.x == 0) {
         item_ok = decode_tile_item(a, t, wk.q_begin, &item_s) ? 1 : 0;
         done_count = 0;
