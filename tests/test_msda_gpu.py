@@ -327,3 +327,53 @@ def test_c_abi_direct_call_and_error_codes(gpu_device):
                                  d.sampling_locations.data_ptr(), d.attention_weights.data_ptr(), out.data_ptr(),
                                  out.data_ptr(), out.data_ptr(), out.data_ptr(), None, 0, 1, bs, nk, nh, hd, nl, nl,
                                  nq, npts, 0, stream) == -4
+
+
+def _backward_c_abi(d, flags, grad_value):
+    """One raw mxd_msda_backward call (float32) on device inputs d; returns (grad_loc, grad_attn)."""
+    lib = _lib.load()
+    shapes, lsi = d.spatial_shapes.int().contiguous(), d.level_start_index.int().contiguous()
+    bs, nk, nh, hd = d.value.shape
+    _, nq, _, nl, npts, _ = d.sampling_locations.shape
+    gl, ga = torch.empty_like(d.sampling_locations), torch.empty_like(d.attention_weights)
+    dims = (bs, nk, nh, hd, nl, nl, nq, npts)
+    nbytes = lib.mxd_msda_backward_workspace_bytes(0, *dims)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=d.value.device)
+    rc = lib.mxd_msda_backward(d.value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), d.sampling_locations.data_ptr(),
+                               d.attention_weights.data_ptr(), d.grad_output.data_ptr(), grad_value.data_ptr(),
+                               gl.data_ptr(), ga.data_ptr(), ws.data_ptr(), nbytes, 0, *dims, flags,
+                               torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    return gl, ga
+
+
+@pytest.mark.parametrize("name,scale", [("tiny", 1.0), ("detr_encoder_bwd", 0.25)])
+def test_backward_accumulate_flag_adds_into_grad_value(gpu_device, name, scale):
+    """MXD_BWD_ACCUMULATE: the image keeps its contents and the gradient is added to it, twice in a row."""
+    inp = workloads.make_inputs(name, with_grad_output=True, scale_queries=scale)
+    ref_gv = oracle_all(inp)[1]
+    d = to_device(inp, gpu_device)
+    gv = torch.full_like(d.value, 0.5)
+    _backward_c_abi(d, _lib.BWD_ACCUMULATE, gv)
+    assert rel_err(gv.double().cpu().numpy(), 0.5 + ref_gv) <= BWD_FP32
+    _backward_c_abi(d, _lib.BWD_ACCUMULATE, gv)
+    assert rel_err(gv.double().cpu().numpy(), 0.5 + 2 * ref_gv) <= BWD_FP32
+    _backward_c_abi(d, 0, gv)  # without the flag the image is overwritten
+    assert rel_err(gv.double().cpu().numpy(), ref_gv) <= BWD_FP32
+
+
+@pytest.mark.parametrize("env", [{"MXD_MSDA_BWD_ATOMIC": "1"}, {"MXD_MSDA_BWD_TILE_Q": "64"},
+                                 {"MXD_MSDA_BWD_TILE_Q": "256"}, {"MXD_MSDA_TILE_TARGET": "128"},
+                                 {"MXD_MSDA_TILE_TARGET": "1000000"}, {"MXD_MSDA_XCD_MODE": "0"}],
+                         ids=lambda e: ",".join(f"{k[9:]}={v}" for k, v in e.items()))
+def test_backward_launch_variants_agree_with_the_oracle(gpu_device, monkeypatch, env):
+    """The tuning knobs read at call time select other code paths (one-kernel atomic backward, other
+    workgroup sizes of the first kernel, tiles split into very many or no query chunks, plain workgroup
+    mapping); every one of them must give the same gradients."""
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    for name, scale in (("tiny", 1.0), ("detr_encoder_bwd", 0.25)):
+        inp = workloads.make_inputs(name, with_grad_output=True, scale_queries=scale)
+        errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+        print(env, name, errs)
