@@ -115,12 +115,13 @@ int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int
                      int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
                      void* hip_stream);
 
-/* Bytes of scratch mxd_msda_backward needs (0 if the sizes are invalid).  It holds one int32
- * key per sample (bs*nh*nl*nq*np*4 bytes, the pixel index of the sample's top-left corner,
- * written by the first backward kernel and scanned by the second) and, for fp16/bf16, an fp32
- * image of grad_value (bs*nk*nh*hd*4) that the sums are formed in before one rounding pass
- * (the reference keeps the same fp32 buffer, MultiScaleDeformableAttn.cpp:93,103-113; its
- * launcher also allocates a workspace per call, include/csrc/OpApiCommon.h:589-595). */
+/* Bytes of scratch mxd_msda_backward needs (0 if the sizes are invalid, and for float32 sizes
+ * that take the one-kernel path with global atomics).  It holds the hand-over between the two
+ * backward kernels -- a table of run starts and two 16-byte records per sample, written
+ * sorted by tile by the first kernel and streamed by the second -- and, for fp16/bf16, an
+ * fp32 image of grad_value (bs*nk*nh*hd*4) that the sums are formed in before one rounding
+ * pass (the reference keeps the same fp32 buffer, MultiScaleDeformableAttn.cpp:93,103-113;
+ * its launcher also allocates a workspace per call, include/csrc/OpApiCommon.h:589-595). */
 size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
                                          int64_t nl_attn, int64_t nq, int64_t np);
 
@@ -133,7 +134,8 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
  * zero-fills the fp32 accumulation image of grad_value (grad_value itself for fp32, the
  * workspace otherwise; skipped under MXD_BWD_ACCUMULATE), runs the gradient kernels, and for
  * fp16/bf16 rounds the image into grad_value.  Every element of the three outputs is written.
- * `workspace` (16-byte aligned, at least mxd_msda_backward_workspace_bytes()) is required. */
+ * `workspace` (16-byte aligned, at least mxd_msda_backward_workspace_bytes()) is required
+ * whenever that size is not 0. */
 int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
                       const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
                       void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype,
