@@ -112,3 +112,51 @@ def multi_scale_deformable_attn_backward(value, shape, level_start_index, locati
                                    nh, hd, nl, nl_attn, nq, npts, 0, stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return grad_value, grad_loc, grad_attn
+
+
+def msda_fused_forward(value, value_spatial_shapes, value_level_start_index, reference_points, sampling_offsets,
+                       attention_logits):
+    """Forward of the operator with the callers' softmax and sampling-location arithmetic folded into the
+    kernel (``mxd_msda_fused_forward``): reference_points ``[bs, nq, nl, 2|4]``, sampling_offsets
+    ``[bs, nq, nh, nl, np, 2]``, attention_logits ``[bs, nq, nh, nl*np]``.  Returns ``[bs, nq, nh*hd]``."""
+    _check(value.dtype in _FLOAT_CODES,
+           f"value: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {value.dtype}")
+    _check(value_spatial_shapes.dtype == torch.int32 and value_level_start_index.dtype == torch.int32,
+           "value_spatial_shapes / value_level_start_index: int32 tensors expected")
+    _check(value.dim() == 4, "value: expected [bs, num_keys, num_heads, embed_dims]")
+    _check(sampling_offsets.dim() == 6 and sampling_offsets.size(5) == 2,
+           "sampling_offsets: expected [bs, num_queries, num_heads, num_levels, num_points, 2]")
+    bs, nk, nh, hd = value.shape
+    _, nq, _, nl, npts, _ = sampling_offsets.shape
+    _check(value_spatial_shapes.dim() == 2 and tuple(value_spatial_shapes.shape) == (nl, 2),
+           "value_spatial_shapes: expected [num_levels, 2] with the levels of sampling_offsets")
+    _check(value_level_start_index.numel() == nl, "value_level_start_index: expected [num_levels]")
+    _check(sampling_offsets.size(0) == bs and sampling_offsets.size(2) == nh,
+           "sampling_offsets: batch size / num_heads do not match value")
+    _check(reference_points.dim() == 4 and tuple(reference_points.shape[:3]) == (bs, nq, nl),
+           "reference_points: expected [bs, num_queries, num_levels, 2 or 4]")
+    _check(reference_points.size(3) in (2, 4),
+           f"Last dim of reference_points must be 2 or 4, but get {reference_points.size(3)} instead.")
+    _check(attention_logits.numel() == bs * nq * nh * nl * npts and attention_logits.size(0) == bs,
+           "attention_logits: expected [bs, num_queries, num_heads, num_levels*num_points]")
+    _check(value.size(3) <= 256, "The number of embedding dimensions should be less than or equal to 256")
+    tensors = (value, value_spatial_shapes, value_level_start_index, reference_points, sampling_offsets,
+               attention_logits)
+    _check(all(t.is_cuda for t in tensors),
+           "msda_fused_forward: all tensors must live on a GPU (this build has no CPU implementation)")
+    _check(all(t.device == value.device for t in tensors), "msda_fused_forward: tensors are on different devices")
+    lib = _lib.load()
+    dt = value.dtype
+    value = value.contiguous()
+    shapes, lsi = value_spatial_shapes.contiguous(), value_level_start_index.contiguous()
+    ref = reference_points.to(dt).contiguous()
+    off = sampling_offsets.to(dt).contiguous()
+    logits = attention_logits.to(dt).contiguous()
+    output = torch.empty((bs, nq, nh * hd), dtype=dt, device=value.device)
+    with torch.cuda.device(value.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.mxd_msda_fused_forward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), ref.data_ptr(),
+                                        reference_points.size(3), off.data_ptr(), logits.data_ptr(),
+                                        output.data_ptr(), _FLOAT_CODES[dt], bs, nk, nh, hd, nl, nq, npts, stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return output

@@ -17,7 +17,14 @@ from .ops.multi_scale_deformable_attn import (  # noqa: F401
     npu_multi_scale_deformable_attn_function,
 )
 
+from .ops.msda_fused import (  # noqa: F401,E402
+    MultiScaleDeformableAttnFusedFunction,
+    multi_scale_deformable_attn_fused,
+)
+
 __all__ = [
+    "MultiScaleDeformableAttnFusedFunction",
+    "multi_scale_deformable_attn_fused",
     "MultiScaleDeformableAttnFunction",
     "multi_scale_deformable_attn",
     "npu_multi_scale_deformable_attn_function",

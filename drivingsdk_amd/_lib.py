@@ -19,6 +19,7 @@ EXPORTS = (
     "mxd_msda_make_plan",
     "mxd_msda_decode_block",
     "mxd_msda_forward",
+    "mxd_msda_fused_forward",
     "mxd_msda_backward_workspace_bytes",
     "mxd_msda_backward",
 )
@@ -62,6 +63,8 @@ def load():
                                           ctypes.POINTER(ctypes.c_int32 * 4)]
     lib.mxd_msda_forward.restype = ci
     lib.mxd_msda_forward.argtypes = [p] * 6 + [ci] + [i64] * 8 + [p]
+    lib.mxd_msda_fused_forward.restype = ci
+    lib.mxd_msda_fused_forward.argtypes = [p] * 4 + [ci] + [p] * 3 + [ci] + [i64] * 7 + [p]
     lib.mxd_msda_backward_workspace_bytes.restype = ctypes.c_size_t
     lib.mxd_msda_backward_workspace_bytes.argtypes = [ci] + [i64] * 8
     lib.mxd_msda_backward.restype = ci

@@ -204,6 +204,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     if (backward) per_unit += mxd::kChunk * sizeof(mxd::f32x4);
     p->lds_bytes = (uint32_t)(mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)p->waves_per_block * p->units_per_wave * per_unit);
     if (backward && L.tiles) p->lds_bytes += (uint32_t)((mxd::kMaxLevels + L.tbl_stride) * sizeof(int32_t));
+    if (!backward) p->lds_bytes += (uint32_t)(p->waves_per_block * p->units_per_wave * 2 * sizeof(float));  // softmax statistics (fused form)
     return MXD_OK;
 }
 
@@ -286,6 +287,38 @@ int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int
     a.out = output;
     const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_forward: launch failed: %s", hipGetErrorString(e));
+    return MXD_OK;
+}
+
+int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                           const void* reference_points, int ref_dim, const void* sampling_offsets,
+                           const void* attn_logits, void* output, int dtype, int64_t bs, int64_t nk, int64_t nh,
+                           int64_t hd, int64_t nl, int64_t nq, int64_t np, void* hip_stream)
+{
+    const Dims d{bs, nk, nh, hd, nl, nl, nq, np};
+    int rc = check_dims(dtype, d);
+    if (rc != MXD_OK) return rc;
+    if (!value || !spatial_shapes || !level_start_index || !reference_points || !sampling_offsets || !attn_logits || !output)
+        return fail(MXD_E_NULL, "mxd_msda_fused_forward: NULL data pointer");
+    if (ref_dim != 2 && ref_dim != 4)
+        return fail(MXD_E_SHAPE, "Last dim of reference_points must be 2 or 4, but get %d instead.", ref_dim);
+    int align = ptr_align(value);
+    if (ptr_align(output) < align) align = ptr_align(output);
+    mxd::KArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = make_plan(0, dtype, d, align, &a.plan);
+    if (rc != MXD_OK) return rc;
+    fill_args(&a, dtype, d);
+    a.value = value;
+    a.shapes = spatial_shapes;
+    a.lsi = level_start_index;
+    a.loc = sampling_offsets;
+    a.attn = attn_logits;
+    a.ref = reference_points;
+    a.ref_dim = ref_dim;
+    a.out = output;
+    const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_fused_forward: launch failed: %s", hipGetErrorString(e));
     return MXD_OK;
 }
 

@@ -24,6 +24,10 @@ struct KArgs {
     const void* loc;
     const void* attn;
     void* out;             // forward output
+    // fused forward only: `loc` holds sampling offsets, `attn` holds logits (softmax over nl*np inside
+    // the kernel), and the sampling location is reference point + offset / normaliser
+    const void* ref;       // [bs, nq, nl, ref_dim] reference points
+    int32_t ref_dim;       // 2: (x, y); 4: (x, y, w, h) boxes
     const void* grad_out;  // backward only from here
     float* grad_value;     // fp32 accumulation image of grad_value
     void* grad_loc;

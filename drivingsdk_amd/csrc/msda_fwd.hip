@@ -19,11 +19,18 @@
 //     corner outside the image gets an out-of-range offset and the hardware returns zeros,
 //     so zero padding costs no branch and never touches memory (NaNs in unrelated pixels
 //     cannot leak in).
+//
+// FUSED = true folds the two steps that deformable-attention modules run before the operator
+// (Deformable-DETR's MSDeformAttn.forward, mmcv's MultiScaleDeformableAttention.forward) into
+// the geometry stage: softmax of the nl*np attention logits of a unit (statistics per unit by
+// the 16 lanes that later own its samples) and sampling location = reference point +
+// offset / (W, H)  [2-d reference points]  or  + offset / np * (w, h) * 0.5  [boxes].
+// The normalised locations and weights then never exist in memory.
 #include "msda_device.h"
 
 namespace mxd {
 
-template <typename T, int VEC, int NPASS>
+template <typename T, int VEC, int NPASS, bool FUSED>
 __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -50,6 +57,9 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
     const int g = lane >> lpr_log2;                 // unit slot of this lane
     const int c = lane & (a.plan.lanes_per_row - 1);  // position inside the row
     Entry* stage = stage_all + wave * (U * kChunkStride);
+    // softmax statistics of the units of this wavefront (fused form): {max, sum of exp}
+    float* stats = reinterpret_cast<float*>(stage_all + a.plan.waves_per_block * (U * kChunkStride)) + wave * (2 * U);
+    const T* ref = static_cast<const T*>(a.ref);
 
     const T* loc = static_cast<const T*>(a.loc);
     const T* attn = static_cast<const T*>(a.attn);
@@ -80,6 +90,27 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
 #pragma unroll
             for (int v = 0; v < VEC; ++v) acc[p][v] = 0.0f;
 
+        if constexpr (FUSED) {
+            // softmax statistics: lanes 16u..16u+15 share unit u, each takes every 16th logit
+            for (int i = lane; i < entries; i += kWave) {
+                const int u = i >> 4, sl = i & (kChunk - 1), q = q0 + u;
+                const T* lg = attn + (((int64_t)wk.b * a.nq + (q < wk.q_end ? q : wk.q_begin)) * a.nh + wk.h) * a.S_full;
+                float m = -__builtin_inff();
+                for (int s = sl; s < a.S; s += kChunk) m = __builtin_fmaxf(m, to_f32(lg[s]));
+#pragma unroll
+                for (int d = 1; d < kChunk; d <<= 1) m = __builtin_fmaxf(m, __shfl_xor(m, d, kWave));
+                float sum = 0.0f;
+                for (int s = sl; s < a.S; s += kChunk) sum += expf(to_f32(lg[s]) - m);
+#pragma unroll
+                for (int d = 1; d < kChunk; d <<= 1) sum += __shfl_xor(sum, d, kWave);
+                if (sl == 0) {
+                    stats[2 * u] = m;
+                    stats[2 * u + 1] = sum;
+                }
+            }
+            wave_lds_sync();
+        }
+
         for (int c0 = 0; c0 < a.S; c0 += kChunk) {
             // ---- geometry: one sample per lane --------------------------------------------
             for (int i = lane; i < entries; i += kWave) {
@@ -94,6 +125,17 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
                     y = to_f32(loc[2 * e + 1]);
                     aw = to_f32(attn[e]);
                     l = (int)(((uint32_t)s * a.np_magic) >> 20);
+                    if constexpr (FUSED) {
+                        const T* rp = ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim;
+                        if (a.ref_dim == 2) {
+                            x = to_f32(rp[0]) + x / (float)lvl[l].y;
+                            y = to_f32(rp[1]) + y / (float)lvl[l].x;
+                        } else {
+                            x = to_f32(rp[0]) + x / (float)a.np * to_f32(rp[2]) * 0.5f;
+                            y = to_f32(rp[1]) + y / (float)a.np * to_f32(rp[3]) * 0.5f;
+                        }
+                        aw = expf(aw - stats[2 * u]) / stats[2 * u + 1];
+                    }
                 }
                 const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active);
                 Entry en;
@@ -144,8 +186,12 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
 template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, hipStream_t stream)
 {
-    hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS>), dim3(a.plan.grid), dim3(a.plan.block), a.plan.lds_bytes,
-                       stream, a);
+    if (a.ref != nullptr)
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, true>), dim3(a.plan.grid), dim3(a.plan.block),
+                           a.plan.lds_bytes, stream, a);
+    else
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, false>), dim3(a.plan.grid), dim3(a.plan.block),
+                           a.plan.lds_bytes, stream, a);
     return hipGetLastError();
 }
 

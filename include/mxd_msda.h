@@ -115,6 +115,22 @@ int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int
                      int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
                      void* hip_stream);
 
+/* Forward with the caller's pre-processing folded in.  No single function of the reference
+ * corresponds to it: it replaces, together, the softmax over the nl*np attention logits, the
+ * sampling-location arithmetic and the operator call of the deformable-attention modules the
+ * reference's model recipes patch (model_examples/Deformable-DETR/Deformable-DETR_npu.patch:626-652,
+ * model_examples/BEVFormer/bev_former_config.patch:404-421):
+ *     attn = softmax(attn_logits[b,q,h,:])                                 [bs,nq,nh,nl*np]
+ *     loc  = ref[b,q,l,:2] + off[b,q,h,l,p,:] / (W_l, H_l)                 ref_dim == 2
+ *     loc  = ref[b,q,l,:2] + off[b,q,h,l,p,:] / np * ref[b,q,l,2:] * 0.5   ref_dim == 4
+ *     output = mxd_msda_forward(value, ..., loc, attn)
+ * reference_points [bs,nq,nl,ref_dim], sampling_offsets [bs,nq,nh,nl,np,2] and attn_logits
+ * [bs,nq,nh,nl*np] have value's dtype; loc and attn are never written to memory. */
+int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                           const void* reference_points, int ref_dim, const void* sampling_offsets,
+                           const void* attn_logits, void* output, int dtype, int64_t bs, int64_t nk, int64_t nh,
+                           int64_t hd, int64_t nl, int64_t nq, int64_t np, void* hip_stream);
+
 /* Bytes of scratch mxd_msda_backward needs (0 if the sizes are invalid, and for float32 sizes
  * that take the one-kernel path with global atomics).  It holds the hand-over between the two
  * backward kernels -- a table of run starts and two 16-byte records per sample, written

@@ -135,3 +135,53 @@ def msda_grid_sample_fwd_bwd(value, shapes, loc, attn, grad_out=None, dtype=torc
         return out.detach(), None, None, None
     out.backward(grad_out.detach().to("cpu", dtype))
     return out.detach(), v.grad, lo.grad, at.grad
+
+
+def fused_sampling_inputs(shapes, reference_points, sampling_offsets, attention_logits):
+    """What deformable-attention modules compute between their linear layers and the operator
+    (model_examples/Deformable-DETR/Deformable-DETR_npu.patch:626-652 of the reference; upstream
+    MSDeformAttn.forward): softmax over the nl*np logits of a (batch, query, head) and
+    location = reference point + offset / (W, H), or + offset / np * (w, h) / 2 for box
+    reference points.  Written with explicit index arithmetic, not by calling the product's helper.
+    Pinned in tests/test_oracle.py by closed forms (zero offsets, uniform logits, a hand case)."""
+    bs, nq, nh, nl, npts, _ = sampling_offsets.shape
+    z = attention_logits.reshape(bs, nq, nh, nl * npts)
+    z = z - z.max(dim=-1, keepdim=True).values
+    e = torch.exp(z)
+    attn = (e / e.sum(dim=-1, keepdim=True)).reshape(bs, nq, nh, nl, npts)
+    loc = []
+    for lvl in range(nl):
+        h, w = float(shapes[lvl, 0]), float(shapes[lvl, 1])
+        ref = reference_points[:, :, lvl]                      # [bs, nq, 2 or 4]
+        off = sampling_offsets[:, :, :, lvl]                   # [bs, nq, nh, np, 2]
+        if reference_points.shape[-1] == 2:
+            x = ref[:, :, None, None, 0] + off[..., 0] / w
+            y = ref[:, :, None, None, 1] + off[..., 1] / h
+        else:
+            x = ref[:, :, None, None, 0] + off[..., 0] / npts * ref[:, :, None, None, 2] * 0.5
+            y = ref[:, :, None, None, 1] + off[..., 1] / npts * ref[:, :, None, None, 3] * 0.5
+        loc.append(torch.stack([x, y], dim=-1))
+    return torch.stack(loc, dim=3), attn
+
+
+def fused_fwd_bwd(value, shapes, reference_points, sampling_offsets, attention_logits, grad_out=None,
+                  dtype=torch.float64, loc_dtype=None):
+    """Fused form through ``msda_grid_sample`` and autograd in ``dtype``.  With ``loc_dtype`` (float32) the
+    sampling locations are first formed in that type -- the same correctly rounded operations in the same order
+    as the callers' torch code and the kernel, hence the same bits -- and only then widened, so that the
+    comparison is not dominated by which side of a cell edge a float32 location falls on.
+    Returns (out, grad_value, grad_reference_points, grad_sampling_offsets, grad_attention_logits)."""
+    g = grad_out is not None
+    v = value.detach().to("cpu", dtype).requires_grad_(g)
+    r = reference_points.detach().to("cpu", dtype).requires_grad_(g)
+    o = sampling_offsets.detach().to("cpu", dtype).requires_grad_(g)
+    z = attention_logits.detach().to("cpu", dtype).requires_grad_(g)
+    sh = shapes.cpu().long()
+    loc, attn = fused_sampling_inputs(sh, r, o, z)
+    if loc_dtype is not None:
+        loc = fused_sampling_inputs(sh, r.to(loc_dtype), o.to(loc_dtype), z.to(loc_dtype))[0].to(dtype)
+    out = msda_grid_sample(v, sh, loc, attn)
+    if not g:
+        return out.detach(), None, None, None, None
+    out.backward(grad_out.detach().to("cpu", dtype))
+    return out.detach(), v.grad, r.grad, o.grad, z.grad

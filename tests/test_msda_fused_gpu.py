@@ -1,0 +1,132 @@
+"""Fused form (softmax + sampling-location arithmetic inside the forward kernel) against the CPU oracle.
+Tolerances as for the plain operator: forward 1e-5, gradients 1e-4 (float32), 2e-3 for 16-bit types."""
+import numpy as np
+import pytest
+import torch
+
+import drivingsdk_amd
+from drivingsdk_amd import _lib, workloads
+from drivingsdk_amd.ops import msda_fused
+from oracle import msda_oracle as orc
+from util import BWD_FP32, FWD_FP32, HALF, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def make_fused_inputs(name, ref_dim=2, scale_queries=1.0, seed=77, dtype=torch.float32):
+    """Module-style inputs on the pyramid of a named workload: reference points in [0,1), offsets of a few
+    pixels, Gaussian logits."""
+    cfg = workloads.WORKLOADS[name]
+    shapes, lsi = workloads.level_tensors(cfg["levels"])
+    g = torch.Generator().manual_seed(seed)
+    nk = int(shapes.prod(1).sum())
+    bs, nh, hd, npts, nl = cfg["bs"], cfg["nh"], cfg["hd"], cfg["np"], shapes.shape[0]
+    nq = max(1, int(round((cfg["nq"] or nk) * scale_queries)))
+    value = torch.randn(bs, nk, nh, hd, generator=g)
+    ref = torch.rand(bs, nq, nl, ref_dim, generator=g)
+    if ref_dim == 4:
+        ref[..., 2:] = ref[..., 2:] * 0.3 + 0.05
+    off = torch.randn(bs, nq, nh, nl, npts, 2, generator=g) * (3.0 if ref_dim == 2 else 1.5)
+    logits = torch.randn(bs, nq, nh, nl * npts, generator=g) * 2.0
+    grad_out = torch.randn(bs, nq, nh * hd, generator=g)
+    return [t.to(dtype) for t in (value,)] + [shapes, lsi] + [t.to(dtype) for t in (ref, off, logits, grad_out)]
+
+
+def _edge_masks(shapes, ref, off, logits):
+    """Samples whose float32 location lies within 2^-20 px of (not on) a cell edge -- the location gradient
+    jumps there -- and the reference points that own such a sample."""
+    loc = orc.fused_sampling_inputs(shapes, ref.float(), off.float(), logits.float())[0].double()
+    near = torch.zeros(loc.shape[:-1], dtype=torch.bool)
+    for lvl, (h, w) in enumerate(shapes.tolist()):
+        w_im = loc[:, :, :, lvl, :, 0] * w - 0.5
+        h_im = loc[:, :, :, lvl, :, 1] * h - 0.5
+        dw, dh = (w_im - w_im.round()).abs(), (h_im - h_im.round()).abs()
+        near[:, :, :, lvl] = ((dw > 0) & (dw < 2.0 ** -20)) | ((dh > 0) & (dh < 2.0 ** -20))
+    ref_near = near.any(dim=4).any(dim=2)                     # [bs, nq, nl]
+    return near.numpy(), ref_near.numpy()
+
+
+def _compare(got, want, shapes, ref, off, logits, tols):
+    near, ref_near = _edge_masks(shapes, ref, off, logits)
+    assert near.mean() < 1e-3
+    keep = {"grad_reference_points": ~ref_near[..., None], "grad_sampling_offsets": ~near[..., None]}
+    names = ("output", "grad_value", "grad_reference_points", "grad_sampling_offsets", "grad_attention_logits")
+    errs = {}
+    for n, g_, w_, tol in zip(names, got, want, tols):
+        w_ = w_.numpy()
+        if n in keep:
+            g_, w_ = g_ * keep[n], w_ * keep[n]
+        errs[n] = rel_err(g_, w_)
+        assert errs[n] <= tol, (n, errs)
+    return errs
+
+
+def _run(value, shapes, lsi, ref, off, logits, grad_out, device):
+    v = value.to(device).requires_grad_()
+    r = ref.to(device).requires_grad_()
+    o = off.to(device).requires_grad_()
+    z = logits.to(device).requires_grad_()
+    out = drivingsdk_amd.multi_scale_deformable_attn_fused(v, shapes.to(device), lsi.to(device), r, o, z)
+    out.backward(grad_out.to(device))
+    return [t.detach().double().cpu().numpy() for t in (out, v.grad, r.grad, o.grad, z.grad)]
+
+
+@pytest.mark.parametrize("name,ref_dim,scale", [("tiny", 2, 1.0), ("tiny", 4, 1.0), ("detr_encoder", 2, 0.25),
+                                                ("bevformer_sca", 2, 0.1)])
+def test_fused_forward_and_gradients_fp32(gpu_device, name, ref_dim, scale):
+    inp = make_fused_inputs(name, ref_dim, scale)
+    value, shapes, lsi, ref, off, logits, grad_out = inp
+    want = orc.fused_fwd_bwd(value, shapes, ref, off, logits, grad_out, loc_dtype=torch.float32)
+    got = _run(*inp, gpu_device)
+    print(name, ref_dim, _compare(got, want, shapes, ref, off, logits, (FWD_FP32,) + (BWD_FP32,) * 4))
+
+
+def test_fused_forward_equals_the_unfused_composition(gpu_device):
+    """Same inputs through torch's softmax / location arithmetic and the plain operator."""
+    inp = make_fused_inputs("detr_encoder", 2, 0.25)
+    value, shapes, lsi, ref, off, logits, _ = [t.to(gpu_device) for t in inp]
+    fused = drivingsdk_amd.multi_scale_deformable_attn_fused(value, shapes, lsi, ref, off, logits)
+    loc, attn = msda_fused.sampling_inputs(shapes, ref, off, logits)
+    plain = drivingsdk_amd.multi_scale_deformable_attn(value, shapes, lsi, loc, attn)
+    assert rel_err(fused.double().cpu().numpy(), plain.double().cpu().numpy()) <= FWD_FP32
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_forward_16bit(gpu_device, dtype):
+    inp = make_fused_inputs("tiny", 2, 1.0, dtype=dtype)
+    value, shapes, lsi, ref, off, logits, _ = inp
+    want = orc.fused_fwd_bwd(value, shapes, ref, off, logits)[0]     # float64 on the rounded inputs
+    out = drivingsdk_amd.multi_scale_deformable_attn_fused(*[t.to(gpu_device) for t in inp[:6]])
+    assert out.dtype == dtype
+    # one rounding of the float32 result to the 16-bit type: float16 within the 16-bit tolerance; a bfloat16
+    # half-ulp is up to 2^-8 of the element itself, which for the largest element is all of this error measure
+    tol = HALF if dtype == torch.float16 else 2.0 ** -8
+    assert rel_err(out.double().cpu().numpy(), want.numpy()) <= tol
+
+
+def test_fused_more_than_16_samples_per_unit_and_many_heads(gpu_device):
+    """nl*np = 32 (two staging chunks, strided softmax statistics), head_dim 16 (16 units per wavefront)."""
+    g = torch.Generator().manual_seed(5)
+    shapes, lsi = workloads.level_tensors(((20, 30), (10, 15), (5, 8), (3, 4)))
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh, hd, nl, npts = 2, 333, 5, 16, 4, 8
+    value = torch.randn(bs, nk, nh, hd, generator=g)
+    ref = torch.rand(bs, nq, nl, 2, generator=g)
+    off = torch.randn(bs, nq, nh, nl, npts, 2, generator=g) * 2
+    logits = torch.randn(bs, nq, nh, nl * npts, generator=g) * 3
+    grad_out = torch.randn(bs, nq, nh * hd, generator=g)
+    want = orc.fused_fwd_bwd(value, shapes, ref, off, logits, grad_out, loc_dtype=torch.float32)
+    got = _run(value, shapes, lsi, ref, off, logits, grad_out, gpu_device)
+    _compare(got, want, shapes, ref, off, logits, (FWD_FP32,) + (BWD_FP32,) * 4)
+
+
+def test_fused_error_paths(gpu_device):
+    inp = make_fused_inputs("tiny", 2, 0.05)
+    value, shapes, lsi, ref, off, logits, _ = [t.to(gpu_device) for t in inp]
+    with pytest.raises(RuntimeError, match="must be 2 or 4"):
+        drivingsdk_amd.multi_scale_deformable_attn_fused(value, shapes, lsi, ref[..., :1].repeat(1, 1, 1, 3), off, logits)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        drivingsdk_amd.multi_scale_deformable_attn_fused(value.cpu(), shapes.cpu(), lsi.cpu(), ref.cpu(), off.cpu(),
+                                                         logits.cpu())
+    lib = _lib.load()
+    assert lib.mxd_msda_fused_forward(None, None, None, None, 2, None, None, None, 0, 1, 10, 1, 8, 1, 1, 1, None) == -3

@@ -235,3 +235,77 @@ def test_tiny_workload_matches_committed_fixture():
     np.testing.assert_allclose(gl.numpy()[0, rows_q], fx["grad_sampling_locations"], rtol=1e-11, atol=1e-12)
     np.testing.assert_allclose(ga.numpy()[0, rows_q], fx["grad_attention_weights"], rtol=1e-12, atol=1e-13)
     np.testing.assert_allclose(float(out.double().sum()), float(fx["output_sum"]), rtol=1e-12)
+
+
+# ---- fused form: softmax + sampling-location arithmetic in front of the operator -------------------
+
+def _fused_case(ref_dim=2, seed=7):
+    g = torch.Generator().manual_seed(seed)
+    shapes = torch.tensor([[6, 5], [3, 4]])
+    lsi = torch.tensor([0, 30])
+    bs, nq, nh, hd, nl, npts = 2, 5, 3, 4, 2, 3
+    value = torch.randn(bs, 42, nh, hd, generator=g, dtype=torch.float64)
+    ref = torch.rand(bs, nq, nl, ref_dim, generator=g, dtype=torch.float64)
+    off = torch.randn(bs, nq, nh, nl, npts, 2, generator=g, dtype=torch.float64)
+    logits = torch.randn(bs, nq, nh, nl * npts, generator=g, dtype=torch.float64)
+    return value, shapes, lsi, ref, off, logits
+
+
+def test_fused_inputs_closed_forms():
+    value, shapes, lsi, ref, off, logits = _fused_case()
+    # zero offsets: every point of a level sits on the reference point; equal logits: weights 1/(nl*np)
+    loc, attn = orc.fused_sampling_inputs(shapes, ref, torch.zeros_like(off), torch.full_like(logits, 3.25))
+    assert torch.equal(loc, ref[:, :, None, :, None, :].expand_as(loc))
+    assert torch.allclose(attn, torch.full_like(attn, 1.0 / 6), rtol=0, atol=1e-15)
+    # one pixel of offset moves the location by 1/W horizontally and 1/H vertically
+    one = torch.ones_like(off)
+    loc, _ = orc.fused_sampling_inputs(shapes, ref, one, logits)
+    for lvl, (h, w) in enumerate(shapes.tolist()):
+        d = loc[:, :, :, lvl] - ref[:, :, None, lvl, None, :]
+        assert torch.allclose(d[..., 0], torch.full_like(d[..., 0], 1.0 / w), rtol=0, atol=1e-15)
+        assert torch.allclose(d[..., 1], torch.full_like(d[..., 1], 1.0 / h), rtol=0, atol=1e-15)
+    # softmax: rows sum to one, are shift invariant, and follow exp ratios
+    _, attn = orc.fused_sampling_inputs(shapes, ref, off, logits)
+    _, attn_shift = orc.fused_sampling_inputs(shapes, ref, off, logits + 11.0)
+    flat = attn.flatten(3)
+    assert torch.allclose(flat.sum(-1), torch.ones_like(flat.sum(-1)), rtol=0, atol=1e-14)
+    assert torch.allclose(attn, attn_shift, rtol=0, atol=1e-14)
+    assert torch.allclose(flat[..., 0] / flat[..., 1], torch.exp(logits[..., 0] - logits[..., 1]), rtol=1e-12)
+    # hand case: logits (0, ln 3) -> weights (1/4, 3/4)
+    lg = torch.tensor([0.0, np.log(3.0)], dtype=torch.float64).view(1, 1, 1, 2)
+    _, a2 = orc.fused_sampling_inputs(torch.tensor([[2, 2]]), torch.zeros(1, 1, 1, 2, dtype=torch.float64),
+                                      torch.zeros(1, 1, 1, 1, 2, 2, dtype=torch.float64), lg)
+    assert torch.allclose(a2.flatten(), torch.tensor([0.25, 0.75], dtype=torch.float64), rtol=0, atol=1e-15)
+
+
+def test_fused_inputs_box_reference_points():
+    value, shapes, lsi, ref, off, logits = _fused_case(ref_dim=4)
+    loc, _ = orc.fused_sampling_inputs(shapes, ref, off, logits)
+    b, q, h, l, p = 1, 3, 2, 1, 2
+    want_x = ref[b, q, l, 0] + off[b, q, h, l, p, 0] / 3 * ref[b, q, l, 2] * 0.5
+    want_y = ref[b, q, l, 1] + off[b, q, h, l, p, 1] / 3 * ref[b, q, l, 3] * 0.5
+    assert loc[b, q, h, l, p, 0] == want_x and loc[b, q, h, l, p, 1] == want_y
+
+
+def test_fused_gradients_by_finite_differences():
+    value, shapes, lsi, ref, off, logits = _fused_case()
+    off = off * 0.3
+    g = torch.Generator().manual_seed(11)
+    grad_out = torch.randn(2, 5, 12, generator=g, dtype=torch.float64)
+    out, gv, gr, go, gz = orc.fused_fwd_bwd(value, shapes, ref, off, logits, grad_out)
+
+    def f(r, o, z):
+        return (orc.fused_fwd_bwd(value, shapes, r, o, z)[0] * grad_out).sum()
+    eps = 1e-6
+    for name, t, gt in (("ref", ref, gr), ("off", off, go), ("logits", logits, gz)):
+        flat = t.flatten()
+        for idx in (0, flat.numel() // 2, flat.numel() - 1):
+            tp, tm = flat.clone(), flat.clone()
+            tp[idx] += eps
+            tm[idx] -= eps
+            args_p = [ref, off, logits]
+            args_m = [ref, off, logits]
+            k = ("ref", "off", "logits").index(name)
+            args_p[k], args_m[k] = tp.view_as(t), tm.view_as(t)
+            fd = (f(*args_p) - f(*args_m)) / (2 * eps)
+            assert abs(fd - gt.flatten()[idx]) <= 1e-5 * max(1.0, abs(fd)), (name, idx, fd, gt.flatten()[idx])
