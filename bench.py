@@ -78,6 +78,35 @@ def _kernel_times(d, iters, warmup):
     return res
 
 
+def _module_forward_times(d, iters, warmup):
+    """The step either side of the operator in the calling module (softmax of the logits, location =
+    reference point + offset / (W, H)): torch element-wise kernels followed by the operator, against the
+    fused forward in which both happen inside the kernel.  Same synthetic module inputs for both."""
+    import torch
+
+    import drivingsdk_amd
+    from drivingsdk_amd.ops import msda_fused
+
+    bs, nk, nh, hd = d.value.shape
+    _, nq, _, nl, npts, _ = d.sampling_locations.shape
+    g = torch.Generator(device="cpu").manual_seed(99)
+    dev = d.value.device
+    ref = torch.rand(bs, nq, nl, 2, generator=g).to(dev)
+    off = (torch.randn(bs, nq, nh, nl, npts, 2, generator=g) * 3.0).to(dev)
+    logits = torch.randn(bs, nq, nh, nl * npts, generator=g).to(dev)
+
+    def unfused():
+        loc, attn = msda_fused.sampling_inputs(d.spatial_shapes, ref, off, logits)
+        return drivingsdk_amd.multi_scale_deformable_attn(d.value, d.spatial_shapes, d.level_start_index, loc, attn)
+
+    def fused():
+        return drivingsdk_amd.multi_scale_deformable_attn_fused(d.value, d.spatial_shapes, d.level_start_index, ref,
+                                                                off, logits)
+
+    with torch.no_grad():
+        return {"unfused_ms": _event_ms(unfused, iters, warmup), "fused_ms": _event_ms(fused, iters, warmup)}
+
+
 def _committed_traffic(workload, dtype):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
     kernel of known size) and committed under profiles/; None when no measurement covers this run."""
@@ -222,6 +251,8 @@ def main():
                     "fwd_plus_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) /
                     ((k["forward_ms"] + k["backward_with_zero_fill_ms"]) * 1e-3) / 1e9},
     }
+    if args.dtype == "float32":
+        result["module_forward"] = _module_forward_times(d, iters=max(args.steps, 50), warmup=max(args.warmup, 10))
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _cpu_baseline(inp)
         result["speedup_vs_cpu_baseline"] = result["value"] / result["cpu_baseline"]["value"]
