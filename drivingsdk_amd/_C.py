@@ -160,3 +160,79 @@ def msda_fused_forward(value, value_spatial_shapes, value_level_start_index, ref
                                         output.data_ptr(), _FLOAT_CODES[dt], bs, nk, nh, hd, nl, nq, npts, stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return output
+
+
+# ---- deformable aggregation (mx_driving/csrc/DeformableAggregation.cpp:20-82 of the reference) --------------
+
+def _dagg_check(mc_ms_feat, spatial_shape, scale_start_index, sampling_location, weights, name):
+    _check(mc_ms_feat.dim() == 3, f"mc_ms_feat.dim() must be 3, but got: {mc_ms_feat.dim()}")
+    _check(spatial_shape.dim() == 3, f"spatial_shape.dim() must be 3, but got: {spatial_shape.dim()}")
+    _check(scale_start_index.dim() == 2, f"scale_start_index.dim() must be 2, but got: {scale_start_index.dim()}")
+    _check(sampling_location.dim() == 5, f"sampling_location.dim() must be 5, but got: {sampling_location.dim()}")
+    _check(weights.dim() == 6, f"weights.dim() must be 6, but got: {weights.dim()}")
+    _check(mc_ms_feat.dtype in _FLOAT_CODES,
+           f"mc_ms_feat: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {mc_ms_feat.dtype}")
+    _check(spatial_shape.dtype == torch.int32 and scale_start_index.dtype == torch.int32,
+           "spatial_shape / scale_start_index: int32 tensors expected")
+    bs, num_feat, num_embeds = mc_ms_feat.shape
+    _, num_anchors, num_pts, num_cams, num_scale, num_groups = weights.shape
+    _check(weights.size(0) == bs, "weights: batch size does not match mc_ms_feat")
+    _check(tuple(spatial_shape.shape) == (num_cams, num_scale, 2), "spatial_shape: expected [num_cams, num_scale, 2]")
+    _check(tuple(scale_start_index.shape) == (num_cams, num_scale), "scale_start_index: expected [num_cams, num_scale]")
+    _check(tuple(sampling_location.shape) == (bs, num_anchors, num_pts, num_cams, 2),
+           "sampling_location: expected [bs, num_anchors, num_pts, num_cams, 2]")
+    _check(num_groups > 0 and num_embeds % num_groups == 0, "num_embeds must be a multiple of weights.sizes()[5]")
+    tensors = (mc_ms_feat, spatial_shape, scale_start_index, sampling_location, weights)
+    _check(all(t.is_cuda for t in tensors),
+           f"{name}: all tensors must live on a GPU (this build has no CPU implementation)")
+    _check(all(t.device == mc_ms_feat.device for t in tensors), f"{name}: tensors are on different devices")
+    return bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups
+
+
+def deformable_aggregation(mc_ms_feat, spatial_shape, scale_start_index, sampling_location, weights):
+    """Forward.  Returns ``[bs, num_anchors, num_embeds]`` in mc_ms_feat's dtype."""
+    dims = _dagg_check(mc_ms_feat, spatial_shape, scale_start_index, sampling_location, weights,
+                       "deformable_aggregation")
+    lib = _lib.load()
+    dt = mc_ms_feat.dtype
+    feat = mc_ms_feat.contiguous()
+    ss, si = spatial_shape.contiguous(), scale_start_index.contiguous()
+    loc, w = sampling_location.to(dt).contiguous(), weights.to(dt).contiguous()
+    out = torch.empty((dims[0], dims[5], dims[2]), dtype=dt, device=feat.device)
+    with torch.cuda.device(feat.device):
+        rc = lib.mxd_dagg_forward(feat.data_ptr(), ss.data_ptr(), si.data_ptr(), loc.data_ptr(), w.data_ptr(),
+                                  out.data_ptr(), _FLOAT_CODES[dt], *dims, torch.cuda.current_stream().cuda_stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return out
+
+
+def deformable_aggregation_backward(mc_ms_feat, spatial_shape, scale_start_index, sampling_location, weights,
+                                    grad_output, grad_mc_ms_feat=None, grad_sampling_location=None, grad_weights=None):
+    """Backward.  Returns (grad_mc_ms_feat, grad_sampling_location, grad_weights).  The three optional
+    tensors are the pre-allocated outputs the reference's binding takes; they are overwritten when given
+    (contiguous, of the inputs' shapes and dtype) and allocated otherwise."""
+    dims = _dagg_check(mc_ms_feat, spatial_shape, scale_start_index, sampling_location, weights,
+                       "deformable_aggregation_backward")
+    _check(grad_output.is_cuda and grad_output.device == mc_ms_feat.device, "grad_output must be on the inputs' GPU")
+    _check(tuple(grad_output.shape) == (dims[0], dims[5], dims[2]), "grad_output: expected [bs, num_anchors, num_embeds]")
+    lib = _lib.load()
+    dt = mc_ms_feat.dtype
+    feat = mc_ms_feat.contiguous()
+    ss, si = spatial_shape.contiguous(), scale_start_index.contiguous()
+    loc, w = sampling_location.to(dt).contiguous(), weights.to(dt).contiguous()
+    go = grad_output.to(dt).contiguous()
+
+    def out_like(given, like):
+        ok = given is not None and given.is_contiguous() and given.dtype == dt and given.shape == like.shape \
+            and given.device == like.device
+        return given if ok else torch.empty_like(like)
+    gf, gl, gw = out_like(grad_mc_ms_feat, feat), out_like(grad_sampling_location, loc), out_like(grad_weights, w)
+    code = _FLOAT_CODES[dt]
+    nbytes = lib.mxd_dagg_backward_workspace_bytes(code, *dims)
+    workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=feat.device)
+    with torch.cuda.device(feat.device):
+        rc = lib.mxd_dagg_backward(feat.data_ptr(), ss.data_ptr(), si.data_ptr(), loc.data_ptr(), w.data_ptr(),
+                                   go.data_ptr(), gf.data_ptr(), gl.data_ptr(), gw.data_ptr(), workspace.data_ptr(),
+                                   nbytes, code, *dims, torch.cuda.current_stream().cuda_stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return gf, gl, gw

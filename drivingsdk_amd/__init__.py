@@ -17,12 +17,20 @@ from .ops.multi_scale_deformable_attn import (  # noqa: F401
     npu_multi_scale_deformable_attn_function,
 )
 
+from .ops.deformable_aggregation import (  # noqa: F401,E402
+    AdsDeformableAggregation,
+    deformable_aggregation,
+    npu_deformable_aggregation,
+)
 from .ops.msda_fused import (  # noqa: F401,E402
     MultiScaleDeformableAttnFusedFunction,
     multi_scale_deformable_attn_fused,
 )
 
 __all__ = [
+    "AdsDeformableAggregation",
+    "deformable_aggregation",
+    "npu_deformable_aggregation",
     "MultiScaleDeformableAttnFusedFunction",
     "multi_scale_deformable_attn_fused",
     "MultiScaleDeformableAttnFunction",

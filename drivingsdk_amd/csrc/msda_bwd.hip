@@ -30,7 +30,7 @@
 
 namespace mxd {
 
-template <typename T, int VEC, int NPASS, bool SCATTER>
+template <typename T, int VEC, int NPASS, bool SCATTER, int SRC>
 __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
     constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
@@ -76,9 +76,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         const int n = (wk.q_end - wk.q_begin) * a.S;
         for (int i = threadIdx.x; i < n; i += blockDim.x) {
             const int qr = i / a.S, s = i - qr * a.S;
-            const int64_t e = (((int64_t)wk.b * a.nq + wk.q_begin + qr) * a.nh + wk.h) * a.S_full + s;
-            const int l = (int)(((uint32_t)s * a.np_magic) >> 20);
-            const Sample sm = sample_geometry(to_f32(loc0[2 * e]), to_f32(loc0[2 * e + 1]), lvl[l], a.nk, true);
+            const SampleRef sr = sample_ref<SRC>(a, wk.b, wk.q_begin + qr, wk.h, s);
+            const int l = sr.l;
+            const float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
+            const bool inside = SRC != kSrcDagg || (cx > 0.0f && cx < 1.0f && cy > 0.0f && cy < 1.0f);
+            const Sample sm = sample_geometry(cx, cy, lvl[l], a.nk, inside);
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
                 if (sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) {
@@ -175,13 +177,14 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 float x = 0.f, y = 0.f, aw = 0.f;
                 int l = 0;
                 if (active) {
-                    const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;
-                    x = to_f32(loc[2 * e]);
-                    y = to_f32(loc[2 * e + 1]);
-                    aw = to_f32(attn[e]);
-                    l = (int)(((uint32_t)s * a.np_magic) >> 20);
+                    const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
+                    x = to_f32(loc[2 * sr.loc_e]);
+                    y = to_f32(loc[2 * sr.loc_e + 1]);
+                    aw = to_f32(attn[sr.w_e]);
+                    l = sr.l;
                 }
-                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active);
+                const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
+                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active && inside);
                 Entry en;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -253,12 +256,13 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 const int u = i >> 4, sl = i & (kChunk - 1);
                 const int s = c0 + sl, q = q0 + u;
                 if ((q < wk.q_end) && (s < a.S)) {
-                    const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;
-                    const float x = to_f32(loc[2 * e]);
-                    const float y = to_f32(loc[2 * e + 1]);
-                    const float aw = to_f32(attn[e]);
-                    const int l = (int)(((uint32_t)s * a.np_magic) >> 20);
-                    const Sample sm = sample_geometry(x, y, lvl[l], a.nk, true);
+                    const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
+                    const float x = to_f32(loc[2 * sr.loc_e]);
+                    const float y = to_f32(loc[2 * sr.loc_e + 1]);
+                    const float aw = to_f32(attn[sr.w_e]);
+                    const int l = sr.l;
+                    const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
+                    const Sample sm = sample_geometry(x, y, lvl[l], a.nk, inside);
                     const f32x4 dd = dots[u * kChunk + sl];
                     float ga = 0.f, gx = 0.f, gy = 0.f;
                     if (sm.valid) {
@@ -267,9 +271,30 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         gx = sm.Wf * aw * (hh * (dd[1] - dd[0]) + sm.lh * (dd[3] - dd[2]));
                         gy = sm.Hf * aw * (hw * (dd[2] - dd[0]) + sm.lw * (dd[3] - dd[1]));
                     }
-                    gattn[e] = from_f32<T>(ga);
-                    gloc[2 * e] = from_f32<T>(gx);
-                    gloc[2 * e + 1] = from_f32<T>(gy);
+                    gattn[sr.w_e] = from_f32<T>(ga);
+                    if constexpr (SRC == kSrcDagg) {
+                        // one location serves the scales of its camera and every head: sum over the
+                        // scales here (neighbouring lanes), per head into a float32 partial image that a
+                        // small kernel adds up over the heads afterwards
+                        float* part = reinterpret_cast<float*>(a.grad_loc) +
+                                      2 * ((int64_t)wk.h * ((int64_t)a.bs * a.nq * a.np * a.cams) + sr.loc_e);
+                        if (a.sc_pow2) {
+                            for (int d = 1; d < a.scales; d <<= 1) {
+                                gx += __shfl_xor(gx, d, kWave);
+                                gy += __shfl_xor(gy, d, kWave);
+                            }
+                            if ((l & (a.scales - 1)) == 0) {
+                                part[0] = gx;
+                                part[1] = gy;
+                            }
+                        } else {
+                            unsafeAtomicAdd(part, gx);
+                            unsafeAtomicAdd(part + 1, gy);
+                        }
+                    } else {
+                        gloc[2 * sr.loc_e] = from_f32<T>(gx);
+                        gloc[2 * sr.loc_e + 1] = from_f32<T>(gy);
+                    }
                     if constexpr (!SCATTER) {
                         // pair records for the tile pass (same decisions as in the counting sweep)
 #pragma unroll
@@ -330,6 +355,35 @@ __global__ __launch_bounds__(256) void msda_round_kernel(const float* src, T* ds
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = from_f32<T>(src[i]);
 }
 
+// deformable aggregation: grad_location[i] = sum over heads of the per-head partial images
+template <typename T>
+__global__ __launch_bounds__(256) void dagg_sum_heads_kernel(const float* part, T* dst, size_t n, int nh)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        float s = 0.0f;
+        for (int h = 0; h < nh; ++h) s += part[(size_t)h * n + i];
+        dst[i] = from_f32<T>(s);
+    }
+}
+
+hipError_t launch_sum_heads(int dtype, const float* part, void* dst, size_t n, int nh, hipStream_t stream)
+{
+    if (n == 0) return hipSuccess;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    const dim3 grid((unsigned)blocks), block(256);
+    if (dtype == MXD_DTYPE_F32)
+        hipLaunchKernelGGL(dagg_sum_heads_kernel<float>, grid, block, 0, stream, part, static_cast<float*>(dst), n, nh);
+    else if (dtype == MXD_DTYPE_F16)
+        hipLaunchKernelGGL(dagg_sum_heads_kernel<f16_t>, grid, block, 0, stream, part, static_cast<f16_t*>(dst), n, nh);
+    else if (dtype == MXD_DTYPE_BF16)
+        hipLaunchKernelGGL(dagg_sum_heads_kernel<bf16_t>, grid, block, 0, stream, part, static_cast<bf16_t*>(dst), n, nh);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t stream)
 {
     if (n == 0) return hipSuccess;
@@ -361,12 +415,18 @@ hipError_t launch_round(int dtype, const float* src, void* dst, size_t n, hipStr
 template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
 {
-    if (scatter)
-        hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true>), dim3(a.plan.grid), dim3(a.plan.block),
-                           a.plan.lds_bytes, stream, a);
-    else
-        hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false>), dim3(a.plan.grid), dim3(a.plan.block),
-                           a.plan.lds_bytes, stream, a);
+    const dim3 grid(a.plan.grid), block(a.plan.block);
+    if (a.cams > 0) {
+        if (scatter)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcDagg>), grid, block, a.plan.lds_bytes, stream, a);
+        else
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcDagg>), grid, block, a.plan.lds_bytes, stream, a);
+    } else {
+        if (scatter)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcPlain>), grid, block, a.plan.lds_bytes, stream, a);
+        else
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcPlain>), grid, block, a.plan.lds_bytes, stream, a);
+    }
     return hipGetLastError();
 }
 

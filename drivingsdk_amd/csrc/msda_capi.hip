@@ -14,6 +14,7 @@ hipError_t launch_backward(int dtype, const KArgs& a, bool scatter, hipStream_t 
 hipError_t launch_gradv_tiles(int dtype, const KArgs& a, const TileArgs& t, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t stream);
 hipError_t launch_round(int dtype, const float* src, void* dst, size_t n, hipStream_t stream);
+hipError_t launch_sum_heads(int dtype, const float* part, void* dst, size_t n, int nh, hipStream_t stream);
 }  // namespace mxd
 
 namespace {
@@ -234,6 +235,39 @@ void fill_args(mxd::KArgs* a, int dtype, const Dims& d)
     a->gbatch_bytes = (uint32_t)(d.nk * d.nh * d.hd * 4);
 }
 
+// Deformable aggregation in the terms of the kernels: channel group = head, (camera, scale) = level,
+// anchor = query, points per anchor = points.
+int dagg_dims(int dtype, int64_t bs, int64_t nf, int64_t C, int64_t cams, int64_t scales, int64_t A, int64_t P,
+              int64_t G, Dims* d)
+{
+    if (G <= 0 || cams <= 0 || scales <= 0 || C <= 0)
+        return fail(MXD_E_SHAPE, "Input Tensor can not be a empty Tensor (C=%lld cams=%lld scales=%lld groups=%lld)",
+                    (long long)C, (long long)cams, (long long)scales, (long long)G);
+    if (C % G != 0) return fail(MXD_E_SHAPE, "num_embeds (%lld) must be a multiple of num_groups (%lld)", (long long)C, (long long)G);
+    *d = Dims{bs, nf, G, C / G, cams * scales, cams * scales, A, P};
+    const int rc = check_dims(dtype, *d);
+    if (rc != MXD_OK) return rc;
+    // sample index -> (point, level) by a multiply-shift that is exact while samples * levels < 2^20
+    if (d->nl * d->np * d->nl >= (1 << 20))
+        return fail(MXD_E_SHAPE, "num_pts*(num_cams*num_scale)^2 = %lld is beyond what this build indexes",
+                    (long long)(d->nl * d->np * d->nl));
+    return MXD_OK;
+}
+
+void fill_dagg(mxd::KArgs* a, int64_t cams, int64_t scales)
+{
+    a->cams = (int32_t)cams;
+    a->scales = (int32_t)scales;
+    a->np_magic = (uint32_t)(((1u << 20) + a->nl - 1) / a->nl);  // sample / levels
+    a->sc_magic = (uint32_t)(((1u << 20) + scales - 1) / scales);
+    a->sc_pow2 = (scales & (scales - 1)) == 0 && scales <= 16;
+}
+
+size_t dagg_part_bytes(const Dims& d, int64_t cams)
+{
+    return (size_t)d.nh * d.bs * d.nq * d.np * cams * 2 * sizeof(float);
+}
+
 }  // namespace
 
 extern "C" {
@@ -396,6 +430,118 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
         e = mxd::launch_round(dtype, image, grad_value, n, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: rounding launch failed: %s", hipGetErrorString(e));
     }
+    return MXD_OK;
+}
+
+int mxd_dagg_forward(const void* mc_ms_feat, const int32_t* spatial_shape, const int32_t* scale_start_index,
+                     const void* sampling_location, const void* weights, void* output, int dtype, int64_t bs,
+                     int64_t num_feat, int64_t num_embeds, int64_t num_cams, int64_t num_scale, int64_t num_anchors,
+                     int64_t num_pts, int64_t num_groups, void* hip_stream)
+{
+    Dims d;
+    int rc = dagg_dims(dtype, bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups, &d);
+    if (rc != MXD_OK) return rc;
+    if (!mc_ms_feat || !spatial_shape || !scale_start_index || !sampling_location || !weights || !output)
+        return fail(MXD_E_NULL, "mxd_dagg_forward: NULL data pointer");
+    int align = ptr_align(mc_ms_feat);
+    if (ptr_align(output) < align) align = ptr_align(output);
+    mxd::KArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = make_plan(0, dtype, d, align, &a.plan);
+    if (rc != MXD_OK) return rc;
+    fill_args(&a, dtype, d);
+    fill_dagg(&a, num_cams, num_scale);
+    a.value = mc_ms_feat;
+    a.shapes = spatial_shape;
+    a.lsi = scale_start_index;
+    a.loc = sampling_location;
+    a.attn = weights;
+    a.out = output;
+    const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_forward: launch failed: %s", hipGetErrorString(e));
+    return MXD_OK;
+}
+
+size_t mxd_dagg_backward_workspace_bytes(int dtype, int64_t bs, int64_t num_feat, int64_t num_embeds, int64_t num_cams,
+                                         int64_t num_scale, int64_t num_anchors, int64_t num_pts, int64_t num_groups)
+{
+    Dims d;
+    if (dagg_dims(dtype, bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups, &d) != MXD_OK)
+        return 0;
+    return bwd_layout(dtype, d).total + dagg_part_bytes(d, num_cams);
+}
+
+int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, const int32_t* scale_start_index,
+                      const void* sampling_location, const void* weights, const void* grad_output,
+                      void* grad_mc_ms_feat, void* grad_sampling_location, void* grad_weights, void* workspace,
+                      size_t workspace_bytes, int dtype, int64_t bs, int64_t num_feat, int64_t num_embeds,
+                      int64_t num_cams, int64_t num_scale, int64_t num_anchors, int64_t num_pts, int64_t num_groups,
+                      void* hip_stream)
+{
+    Dims d;
+    int rc = dagg_dims(dtype, bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups, &d);
+    if (rc != MXD_OK) return rc;
+    if (!mc_ms_feat || !spatial_shape || !scale_start_index || !sampling_location || !weights || !grad_output ||
+        !grad_mc_ms_feat || !grad_sampling_location || !grad_weights)
+        return fail(MXD_E_NULL, "mxd_dagg_backward: NULL data pointer");
+    const BwdLayout L = bwd_layout(dtype, d);
+    const size_t part_bytes = dagg_part_bytes(d, num_cams);
+    const size_t need = L.total + part_bytes;
+    if (!workspace || workspace_bytes < need)
+        return fail(MXD_E_WORKSPACE, "mxd_dagg_backward: workspace of %zu bytes required, %zu given", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u)
+        return fail(MXD_E_WORKSPACE, "mxd_dagg_backward: workspace must be 16-byte aligned");
+    const bool half = elem_size(dtype) == 2;
+    char* ws = static_cast<char*>(workspace);
+    float* image = half ? reinterpret_cast<float*>(ws + L.tbl_bytes + L.rec_bytes) : static_cast<float*>(grad_mc_ms_feat);
+    float* part = reinterpret_cast<float*>(ws + L.total);
+    if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_dagg_backward: grad_mc_ms_feat is not 4-byte aligned");
+    int align = ptr_align(mc_ms_feat);
+    if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
+    mxd::KArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = make_plan(1, dtype, d, align, &a.plan);
+    if (rc != MXD_OK) return rc;
+    fill_args(&a, dtype, d);
+    fill_dagg(&a, num_cams, num_scale);
+    a.value = mc_ms_feat;
+    a.shapes = spatial_shape;
+    a.lsi = scale_start_index;
+    a.loc = sampling_location;
+    a.attn = weights;
+    a.grad_out = grad_output;
+    a.grad_value = image;
+    a.tbl = reinterpret_cast<uint32_t*>(ws);
+    a.rec = reinterpret_cast<mxd::u32x4*>(ws + L.tbl_bytes);
+    a.nwg = (int32_t)L.nwg;
+    a.rec_cap = (int32_t)L.rec_cap;
+    a.tbl_stride = (int32_t)L.tbl_stride;
+    a.grad_loc = part;  // per-head partial images, summed below
+    a.grad_attn = grad_weights;
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    const size_t n = (size_t)bs * num_feat * num_embeds;
+    hipError_t e = mxd::launch_fill_zero(image, n, stream);
+    if (e == hipSuccess && !a.sc_pow2) e = mxd::launch_fill_zero(part, part_bytes / sizeof(float), stream);
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: zero-fill launch failed: %s", hipGetErrorString(e));
+    const bool atomic_mode = !L.tiles;
+    e = mxd::launch_backward(dtype, a, atomic_mode, stream);
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: launch failed: %s", hipGetErrorString(e));
+    if (!atomic_mode) {
+        mxd::TileArgs t;
+        rc = make_tile_args(d, L, a.plan.vec, 0, &t);
+        if (rc != MXD_OK) return rc;
+        t.store_vec = (d.hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
+        e = mxd::launch_gradv_tiles(dtype, a, t, stream);
+        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: tile kernel launch failed: %s", hipGetErrorString(e));
+    }
+    if (half) {
+        e = mxd::launch_round(dtype, image, grad_mc_ms_feat, n, stream);
+        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: rounding launch failed: %s", hipGetErrorString(e));
+    }
+    e = mxd::launch_sum_heads(dtype, part, grad_sampling_location, (size_t)bs * num_anchors * num_pts * num_cams * 2,
+                              (int)num_groups, stream);
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: head sum launch failed: %s", hipGetErrorString(e));
     return MXD_OK;
 }
 

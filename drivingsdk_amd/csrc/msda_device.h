@@ -28,6 +28,14 @@ struct KArgs {
     // the kernel), and the sampling location is reference point + offset / normaliser
     const void* ref;       // [bs, nq, nl, ref_dim] reference points
     int32_t ref_dim;       // 2: (x, y); 4: (x, y, w, h) boxes
+    // deformable aggregation only (source = kSrcDagg): a level is a (camera, scale) pair, nl = cams*scales,
+    // np = points per anchor, sample s = point*nl + level; `loc` is [bs, nq, np, cams, 2] (shared by the
+    // scales of a camera and by all heads = channel groups), `attn` is [bs, nq, np, cams, scales, nh]
+    int32_t cams;
+    int32_t scales;
+    uint32_t sc_magic;     // ceil(2^20/scales): level / scales
+    int32_t sc_pow2;       // scales is a power of two that divides 16: location gradients are summed over the
+                           // scales across lanes and stored once; otherwise they are added with atomics
     const void* grad_out;  // backward only from here
     float* grad_value;     // fp32 accumulation image of grad_value
     void* grad_loc;
@@ -51,6 +59,30 @@ struct KArgs {
     uint32_t gbatch_bytes; // nk*nh*hd*4: one batch element of the fp32 grad image
     mxd_msda_plan plan;
 };
+
+// Where a kernel takes the location and the weight of sample s of unit (b, q, h) from.
+enum : int { kSrcPlain = 0, kSrcFused = 1, kSrcDagg = 2 };
+struct SampleRef {
+    int64_t loc_e;  // index of the (x, y) pair
+    int64_t w_e;    // index of the weight
+    int32_t l;      // level
+};
+template <int SRC>
+__device__ inline SampleRef sample_ref(const KArgs& a, int b, int q, int h, int s)
+{
+    SampleRef r;
+    if constexpr (SRC == kSrcDagg) {
+        const int p = (int)(((uint32_t)s * a.np_magic) >> 20);  // s / nl (np_magic is built for the divisor nl here)
+        r.l = s - p * a.nl;
+        const int cam = (int)(((uint32_t)r.l * a.sc_magic) >> 20);
+        r.loc_e = (((int64_t)b * a.nq + q) * a.np + p) * a.cams + cam;
+        r.w_e = (((int64_t)b * a.nq + q) * a.S + s) * a.nh + h;
+    } else {
+        r.loc_e = r.w_e = (((int64_t)b * a.nq + q) * a.nh + h) * a.S_full + s;
+        r.l = (int)(((uint32_t)s * a.np_magic) >> 20);
+    }
+    return r;
+}
 
 // Launch description of the tile-ownership grad_value kernel.
 constexpr int kTileEntCap = 576;  // list entries (16 bytes) per wavefront and round

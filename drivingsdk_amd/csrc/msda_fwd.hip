@@ -26,13 +26,19 @@
 // the 16 lanes that later own its samples) and sampling location = reference point +
 // offset / (W, H)  [2-d reference points]  or  + offset / np * (w, h) * 0.5  [boxes].
 // The normalised locations and weights then never exist in memory.
+//
+// SRC = kSrcDagg is deformable aggregation (reference: mx_driving/ops/npu_deformable_aggregation.py,
+// kernels/deformable_aggregation/): the same sum with a channel group as head, a (camera, scale) pair as
+// level, one location per (anchor, point, camera) shared by scales and groups, weights laid out
+// [.., point, camera, scale, group], and samples counted only strictly inside (0, 1) x (0, 1).
 #include "msda_device.h"
 
 namespace mxd {
 
-template <typename T, int VEC, int NPASS, bool FUSED>
+template <typename T, int VEC, int NPASS, int SRC>
 __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
 {
+    constexpr bool FUSED = SRC == kSrcFused;
     extern __shared__ __align__(16) unsigned char smem[];
     i32x4* lvl = reinterpret_cast<i32x4*>(smem);                               // [kMaxLevels]
     Entry* stage_all = reinterpret_cast<Entry*>(smem + kMaxLevels * sizeof(i32x4));
@@ -120,11 +126,11 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
                 float x = 0.f, y = 0.f, aw = 0.f;
                 int l = 0;
                 if (active) {
-                    const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;
-                    x = to_f32(loc[2 * e]);
-                    y = to_f32(loc[2 * e + 1]);
-                    aw = to_f32(attn[e]);
-                    l = (int)(((uint32_t)s * a.np_magic) >> 20);
+                    const SampleRef r = sample_ref<SRC>(a, wk.b, q, wk.h, s);
+                    x = to_f32(loc[2 * r.loc_e]);
+                    y = to_f32(loc[2 * r.loc_e + 1]);
+                    aw = to_f32(attn[r.w_e]);
+                    l = r.l;
                     if constexpr (FUSED) {
                         const T* rp = ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim;
                         if (a.ref_dim == 2) {
@@ -137,7 +143,9 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
                         aw = expf(aw - stats[2 * u]) / stats[2 * u + 1];
                     }
                 }
-                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active);
+                // deformable aggregation samples only strictly inside the image (0 < x, y < 1)
+                const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
+                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active && inside);
                 Entry en;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -186,11 +194,14 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
 template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, hipStream_t stream)
 {
-    if (a.ref != nullptr)
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, true>), dim3(a.plan.grid), dim3(a.plan.block),
+    if (a.cams > 0)
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcDagg>), dim3(a.plan.grid), dim3(a.plan.block),
+                           a.plan.lds_bytes, stream, a);
+    else if (a.ref != nullptr)
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcFused>), dim3(a.plan.grid), dim3(a.plan.block),
                            a.plan.lds_bytes, stream, a);
     else
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, false>), dim3(a.plan.grid), dim3(a.plan.block),
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain>), dim3(a.plan.grid), dim3(a.plan.block),
                            a.plan.lds_bytes, stream, a);
     return hipGetLastError();
 }

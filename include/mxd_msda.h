@@ -158,6 +158,36 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
                       int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq,
                       int64_t np, int flags, void* hip_stream);
 
+/* ---- deformable aggregation (Sparse4D / SparseDrive feature sampling) ------------------------
+ * Replaces deformable_aggregation / deformable_aggregation_backward
+ * (mx_driving/csrc/DeformableAggregation.cpp:20-82) with the same tensors:
+ *   mc_ms_feat [bs, num_feat, num_embeds]        spatial_shape [num_cams, num_scale, 2] = (H, W), int32
+ *   scale_start_index [num_cams, num_scale], int32
+ *   sampling_location [bs, num_anchors, num_pts, num_cams, 2] = (x, y)
+ *   weights [bs, num_anchors, num_pts, num_cams, num_scale, num_groups]     output [bs, num_anchors, num_embeds]
+ * output[b,a,c] = sum over (pt, cam, scale) of weights[..., group(c)] * bilinear(feat of (cam, scale), location);
+ * a location counts only when 0 < x < 1 and 0 < y < 1; zero padding outside the map.  The same kernels as
+ * multi-scale deformable attention run it (group = head, (camera, scale) = level, anchor = query). */
+int mxd_dagg_forward(const void* mc_ms_feat, const int32_t* spatial_shape, const int32_t* scale_start_index,
+                     const void* sampling_location, const void* weights, void* output, int dtype, int64_t bs,
+                     int64_t num_feat, int64_t num_embeds, int64_t num_cams, int64_t num_scale, int64_t num_anchors,
+                     int64_t num_pts, int64_t num_groups, void* hip_stream);
+
+/* Bytes of scratch mxd_dagg_backward needs (0 if the sizes are invalid): the hand-over between the two
+ * backward kernels, the fp32 image of grad_mc_ms_feat for 16-bit dtypes, and one float32 partial image of
+ * grad_sampling_location per group. */
+size_t mxd_dagg_backward_workspace_bytes(int dtype, int64_t bs, int64_t num_feat, int64_t num_embeds, int64_t num_cams,
+                                         int64_t num_scale, int64_t num_anchors, int64_t num_pts, int64_t num_groups);
+
+/* Every element of the three gradients is written (the reference zero-fills them first,
+ * mx_driving/ops/npu_deformable_aggregation.py:66-68). */
+int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, const int32_t* scale_start_index,
+                      const void* sampling_location, const void* weights, const void* grad_output,
+                      void* grad_mc_ms_feat, void* grad_sampling_location, void* grad_weights, void* workspace,
+                      size_t workspace_bytes, int dtype, int64_t bs, int64_t num_feat, int64_t num_embeds,
+                      int64_t num_cams, int64_t num_scale, int64_t num_anchors, int64_t num_pts, int64_t num_groups,
+                      void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

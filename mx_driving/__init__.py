@@ -7,7 +7,14 @@ from drivingsdk_amd.ops.multi_scale_deformable_attn import (  # noqa: F401
     npu_multi_scale_deformable_attn_function,
 )
 
+from drivingsdk_amd.ops.deformable_aggregation import (  # noqa: F401,E402  (mx_driving/__init__.py:113)
+    deformable_aggregation,
+    npu_deformable_aggregation,
+)
+
 __all__ = [
+    "deformable_aggregation",
+    "npu_deformable_aggregation",
     "MultiScaleDeformableAttnFunction",
     "multi_scale_deformable_attn",
     "npu_multi_scale_deformable_attn_function",
