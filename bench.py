@@ -149,6 +149,68 @@ def _cpu_baseline(inp, max_seconds=25.0):
                       f"torch grid_sample formulation in float32 with {threads} threads"}
 
 
+def _bench_dagg(args):
+    """Deformable aggregation at a Sparse4D-like size (6 cameras x 4 scales of a 256x704 image, 900 anchors x 13
+    points, 256 channels in 8 groups, batch 6): forward + backward through the autograd Function."""
+    import numpy as np
+    import torch
+
+    import mx_driving
+    from oracle import dagg_oracle
+
+    dev = torch.device("cuda", 0)
+    bs, C, G, A, P, cams = 6, 256, 8, 900, 13, 6
+    maps = [(64, 176), (32, 88), (16, 44), (8, 22)]
+    rng = np.random.default_rng(2024)
+    ss = np.array([maps] * cams, dtype=np.int32)
+    sizes = ss.reshape(-1, 2).prod(1)
+    ssi = np.concatenate([[0], np.cumsum(sizes)[:-1]]).reshape(cams, len(maps)).astype(np.int32)
+    nf = int(sizes.sum())
+    feat_c = rng.standard_normal((bs, nf, C)).astype(np.float32)
+    loc_c = (rng.random((bs, A, P, cams, 2)) * 1.2 - 0.1).astype(np.float32)   # ~30 % of the projections miss a camera
+    w_c = rng.random((bs, A, P, cams, len(maps), G)).astype(np.float32)
+    go_c = rng.standard_normal((bs, A, C)).astype(np.float32)
+    feat = torch.from_numpy(feat_c).to(dev).requires_grad_()
+    loc = torch.from_numpy(loc_c).to(dev).requires_grad_()
+    w = torch.from_numpy(w_c).to(dev).requires_grad_()
+    go = torch.from_numpy(go_c).to(dev)
+    ssd, ssid = torch.from_numpy(ss).to(dev), torch.from_numpy(ssi).to(dev)
+
+    def step():
+        feat.grad = loc.grad = w.grad = None
+        mx_driving.deformable_aggregation(feat, ssd, ssid, loc, w).backward(go)
+
+    def fwd():
+        with torch.no_grad():
+            mx_driving.deformable_aggregation(feat, ssd, ssid, loc, w)
+
+    ms_step = _event_ms(step, args.steps, args.warmup)
+    ms_fwd = _event_ms(fwd, args.steps, args.warmup)
+    # every tensor once: feat, loc, weights in, output out (forward); the same again + grad_output in + three gradients out
+    b_fwd = 4 * (feat.numel() + loc.numel() + w.numel() + bs * A * C)
+    b_bwd = 4 * (feat.numel() + loc.numel() + w.numel() + bs * A * C + feat.numel() + loc.numel() + w.numel())
+    result = {"metric": "deformable_aggregation fwd+bwd anchors/s, Sparse4D-like shape", "value": bs * A / (ms_step * 1e-3),
+              "unit": "anchors/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+              "config": {"workload": f"sparse4d_dagg: bs={bs}, anchors={A}, pts={P}, cams={cams}, scales={len(maps)}, "
+                                     f"embeds={C}, groups={G}, num_feat={nf}"},
+              "roofline": {"bound": "hbm", "kernel": "forward + backward kernels of one step", "achieved":
+                           (b_fwd + b_bwd) / (ms_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                           "frac": (b_fwd + b_bwd) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                           "algorithmic_bytes": b_fwd + b_bwd, "kernel_ms": ms_step},
+              "kernels": {"forward_ms": ms_fwd}}
+    if not args.no_cpu_baseline:
+        t0 = time.perf_counter()
+        dagg_oracle.direct_forward(feat_c[:1], ss, ssi, loc_c[:1], w_c[:1], dtype=np.float32)
+        dagg_oracle.direct_backward(feat_c[:1], ss, ssi, loc_c[:1], w_c[:1], go_c[:1], dtype=np.float32)
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": A / dt, "unit": "anchors/s", "cores": os.cpu_count() if False else 1,
+                                  "kind": "port", "ms_per_step": dt * 1e3 * bs,
+                                  "sample": "one batch element (1/6 of the workload), forward (OpenMP) + backward (serial) "
+                                            "of the C restatement in float32; ms_per_step scaled to the full batch"}
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -174,6 +236,8 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     _lib.load()
+    if args.workload == "sparse4d_dagg":
+        return _bench_dagg(args)
     dev = torch.device("cuda", 0)
     dtype = getattr(torch, args.dtype)
     inp = workloads.make_inputs(args.workload, dtype=dtype, with_grad_output=True)

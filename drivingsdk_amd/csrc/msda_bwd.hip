@@ -63,11 +63,15 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         const int64_t wg_row = ((int64_t)wk.b * a.nh + wk.h) * a.nwg + wk.q_begin / a.plan.tile_q;
         slab = a.rec + wg_row * a.rec_cap;
         if (threadIdx.x == 0) {
+            // the run table has room for tbl_stride - 1 tiles, which is every tile when the levels do not
+            // overlap; a level that does not fit (malformed shapes) is left out of grad_value: -1
             int32_t first = 0;
             for (int l = 0; l < a.nl; ++l) {
                 int32_t px;
-                tile_first[l] = first;
-                first += level_tile_count(lvl[l].x, lvl[l].y, lvl[l].z, a.nk, &px);
+                const int32_t nt = level_tile_count(lvl[l].x, lvl[l].y, lvl[l].z, a.nk, &px);
+                const bool fits = first + nt <= a.tbl_stride - 1;
+                tile_first[l] = fits ? first : -1;
+                if (fits) first += nt;
             }
         }
         for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) cursor[i] = 0;
@@ -83,7 +87,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             const Sample sm = sample_geometry(cx, cy, lvl[l], a.nk, inside);
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
-                if (sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) {
+                if ((sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0) {
                     const int32_t key = sm.cvalid[2 * r] ? sm.pix[2 * r] : sm.pix[2 * r + 1];
                     atomicAdd(&cursor[tile_first[l] + ((key - lvl[l].z) >> kTilePxLog2)], 1);
                 }
@@ -300,7 +304,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 #pragma unroll
                         for (int r = 0; r < 2; ++r) {
                             const bool vl = sm.cvalid[2 * r], vr = sm.cvalid[2 * r + 1];
-                            if (vl || vr) {
+                            if ((vl || vr) && tile_first[l] >= 0) {
                                 const int32_t key = vl ? sm.pix[2 * r] : sm.pix[2 * r + 1];
                                 const float wa = (vl ? sm.w[2 * r] : sm.w[2 * r + 1]) * aw;
                                 const float wb = (vl && vr) ? sm.w[2 * r + 1] * aw : 0.0f;

@@ -46,23 +46,31 @@ struct TileItem {
     int32_t exclusive;           // 1: no other workgroup touches this tile
 };
 
-__device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32_t item, TileItem* out)
+// lv_first / lv_nt: scratch of kMaxLevels entries each (first tile and tile count per level).
+__device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32_t item, TileItem* out,
+                                        int32_t* lv_first, int32_t* lv_nt)
 {
+    // Tiles are numbered level by level as in the first kernel; a level that does not fit the run table
+    // (only possible when the levels overlap) has no tiles.
+    int32_t total = 0;
+    for (int l = 0; l < a.nl; ++l) {
+        int32_t P;
+        const int32_t nt = level_tile_count(a.shapes[2 * l], a.shapes[2 * l + 1], a.lsi[l], a.nk, &P);
+        const bool fits = total + nt <= a.tbl_stride - 1;
+        lv_first[l] = total;
+        lv_nt[l] = fits ? nt : 0;
+        if (fits) total += nt;
+    }
     // Items are numbered from the last level to the first: the coarse levels, whose tiles are
     // split into many long-running items, start first and the short items of the fine levels
     // fill the end of the launch.
-    int32_t tiles_after = 0;  // tiles of the levels not yet visited come first in the run table
-    for (int l = 0; l < a.nl; ++l) {
-        int32_t P;
-        tiles_after += level_tile_count(a.shapes[2 * l], a.shapes[2 * l + 1], a.lsi[l], a.nk, &P);
-    }
     int32_t first = 0;
     for (int l = a.nl - 1; l >= 0; --l) {
+        const int32_t nt = lv_nt[l];
+        if (nt == 0) continue;
         const int32_t H = a.shapes[2 * l], W = a.shapes[2 * l + 1], base = a.lsi[l];
         int32_t P;
-        const int32_t nt = level_tile_count(H, W, base, a.nk, &P);
-        if (nt == 0) continue;
-        tiles_after -= nt;  // now the index of this level's first tile
+        level_tile_count(H, W, base, a.nk, &P);
         // two pair records per sample, spread evenly over the tiles of the level
         const int64_t expect = (2 * (int64_t)a.nq * a.np) / nt;
         int64_t chunks = (expect + t.target - 1) / t.target;
@@ -82,7 +90,7 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
             out->p1 = (out->p0 + kTilePx) < (base + P) ? (out->p0 + kTilePx) : (base + P);
             out->w0 = ci * wpc;
             out->w1 = (out->w0 + wpc) < a.nwg ? (out->w0 + wpc) : a.nwg;
-            out->tile = tiles_after + ti;
+            out->tile = lv_first[l] + ti;
             out->exclusive = chunks == 1;
             return true;
         }
@@ -108,6 +116,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     __shared__ uint32_t run_src_all[NW * kWave];
     __shared__ uint32_t run_pre_all[NW * kWave];
     __shared__ TileItem item_s;
+    __shared__ int32_t lv_first[kMaxLevels], lv_nt[kMaxLevels];
     __shared__ int item_ok;
     __shared__ int done_count;
 
@@ -121,7 +130,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         wk.q_begin = (int32_t)(r / a.bs);
     }
     if (threadIdx.x == 0) {
-        item_ok = decode_tile_item(a, t, wk.q_begin, &item_s) ? 1 : 0;
+        item_ok = decode_tile_item(a, t, wk.q_begin, &item_s, lv_first, lv_nt) ? 1 : 0;
         done_count = 0;
     }
     // an empty list points at the dummy entry of the wavefront that owns the pixel

@@ -103,11 +103,18 @@ int64_t fill_xcd_map(mxd_msda_plan* p, int64_t bs, int64_t nh, int64_t ntiles)
 // tile-ownership pass (and then the hand-over buffers between its two kernels) or through
 // global atomics, and where things live in the caller's workspace.
 //   workspace = [run table][pair records][fp32 image of grad_value, 16-bit dtypes only]
-// queries per workgroup of the first kernel (tile pass): 64, 128 or 256
-static int64_t bwd_tile_q()
+// Queries per workgroup of the first backward kernel (tile pass).  Larger workgroups give the tile pass
+// longer runs; with few queries they leave the chip short of workgroups, so the size steps down until the
+// launch has about six workgroups per CU.  64 is the least for rows of up to 64 bytes (16 units per
+// wavefront, 4 wavefronts), 32 otherwise.  MXD_MSDA_BWD_TILE_Q overrides (32/64/128/256).
+static int64_t bwd_tile_q(int dtype, const Dims& d)
 {
-    const int v = env_int("MXD_MSDA_BWD_TILE_Q", 128);
-    return v == 64 || v == 256 ? v : 128;
+    const int64_t least = d.hd * elem_size(dtype) <= 64 ? 64 : 32;
+    const int v = env_int("MXD_MSDA_BWD_TILE_Q", 0);
+    if (v == 32 || v == 64 || v == 128 || v == 256) return v < least ? least : v;
+    for (int64_t tq = 128; tq > least; tq >>= 1)
+        if (d.bs * d.nh * ((d.nq + tq - 1) / tq) >= 6 * 256) return tq;
+    return least;
 }
 struct BwdLayout {
     bool tiles;          // false: one kernel with global atomics
@@ -122,11 +129,12 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
 {
     BwdLayout L;
     memset(&L, 0, sizeof(L));
-    L.tile_q = bwd_tile_q();
+    L.tile_q = bwd_tile_q(dtype, d);
     L.nwg = (d.nq + L.tile_q - 1) / L.tile_q;
     L.rec_cap = 2 * L.tile_q * d.nl * d.np;
-    // a level has at most nk/kTilePx + 1 tiles whatever spatial_shapes says
-    L.tbl_stride = d.nl * (d.nk / mxd::kTilePx + 1) + 1;
+    // tiles per (batch, head) when the levels do not overlap: sum of ceil(pixels/kTilePx) <= nk/kTilePx + nl
+    // (the kernels leave out levels that would not fit, which can only happen for overlapping levels)
+    L.tbl_stride = d.nk / mxd::kTilePx + d.nl + 1;
     const int64_t tbl = d.bs * d.nh * L.nwg * L.tbl_stride * 4;
     L.tiles = env_int("MXD_MSDA_BWD_ATOMIC", 0) == 0 &&
               L.tbl_stride <= 4096 &&                      // counters of the first kernel live in LDS
