@@ -236,3 +236,77 @@ def deformable_aggregation_backward(mc_ms_feat, spatial_shape, scale_start_index
                                    nbytes, code, *dims, torch.cuda.current_stream().cuda_stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return gf, gl, gw
+
+
+# ---- geometric kernel attention (mx_driving/csrc/GeometricKernelAttentionFunc.cpp:33-118 of the reference) ------
+
+_GKA_LOC_TYPES = (torch.float16, torch.float32, torch.int32, torch.int64)
+
+
+def _gka_check(value, spatial_shapes, level_start_index, sampling_locations, attention_weights):
+    _check(value.dtype in _FLOAT_CODES,
+           f"value_map: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {value.dtype}")
+    _check(spatial_shapes.dtype in (torch.int32, torch.int64),
+           f"spatial_spatial_shapes: int32 or int64 tensor expected but got a tensor with dtype: {spatial_shapes.dtype}")
+    _check(level_start_index.dtype in (torch.int32, torch.int64),
+           f"level_start_index: int32 or int64 tensor expected but got a tensor with dtype: {level_start_index.dtype}")
+    _check(sampling_locations.dtype in _GKA_LOC_TYPES or sampling_locations.dtype == torch.bfloat16,
+           "sampling_locations: float16, float32, int32 or int64 tensor expected but got a tensor with dtype: "
+           f"{sampling_locations.dtype}")
+    _check(attention_weights.dtype in _FLOAT_CODES,
+           f"attention_weights: float16 or float32 tensor expected but got a tensor with dtype: {attention_weights.dtype}")
+    _check(value.dim() == 4 and sampling_locations.dim() == 6 and sampling_locations.size(5) == 2 and
+           attention_weights.dim() == 5, "geometric_kernel_attention: expected value [bs, num_keys, num_heads, dim], "
+           "sampling_locations [bs, num_queries, num_heads, num_levels, num_points, 2], attention_weights [.., num_points]")
+    bs, nk, nh, hd = value.shape
+    _, nq, _, nl, npts, _ = sampling_locations.shape
+    _check(tuple(attention_weights.shape) == (bs, nq, nh, nl, npts) and sampling_locations.size(0) == bs and
+           sampling_locations.size(2) == nh, "geometric_kernel_attention: shapes of the tensors do not match")
+    _check(tuple(spatial_shapes.shape) == (nl, 2) and level_start_index.numel() == nl,
+           "geometric_kernel_attention: spatial_shapes [num_levels, 2] / level_start_index [num_levels] expected")
+    tensors = (value, spatial_shapes, level_start_index, sampling_locations, attention_weights)
+    _check(all(t.is_cuda for t in tensors),
+           "geometric_kernel_attention: all tensors must live on a GPU (this build has no CPU implementation)")
+    _check(all(t.device == value.device for t in tensors), "geometric_kernel_attention: tensors are on different devices")
+    return bs, nk, nh, hd, nl, nq, npts
+
+
+def geometric_kernel_attention_forward(value_map, spatial_shapes, level_start_index, sampling_locations,
+                                       attention_weights, output):
+    """Fills ``output`` ``[bs, num_queries, num_heads*dim]`` (the reference's binding has the same out-parameter)."""
+    dims = _gka_check(value_map, spatial_shapes, level_start_index, sampling_locations, attention_weights)
+    lib = _lib.load()
+    dt = value_map.dtype
+    _check(output.is_cuda and output.is_contiguous() and output.dtype == dt and
+           tuple(output.shape) == (dims[0], dims[5], dims[2] * dims[3]),
+           "output: expected a contiguous [bs, num_queries, num_heads*dim] tensor of value's dtype")
+    value = value_map.contiguous()
+    shapes, lsi = spatial_shapes.int().contiguous(), level_start_index.int().contiguous()
+    loc, attn = sampling_locations.to(dt).contiguous(), attention_weights.to(dt).contiguous()
+    with torch.cuda.device(value.device):
+        rc = lib.mxd_gka_forward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(), attn.data_ptr(),
+                                 output.data_ptr(), _FLOAT_CODES[dt], *dims, torch.cuda.current_stream().cuda_stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+
+
+def geometric_kernel_attention_backward(value, spatial_shapes, level_start_index, sampling_locations, attn_weights,
+                                        grad_output):
+    """Returns (grad_value, grad_attn_weights)."""
+    dims = _gka_check(value, spatial_shapes, level_start_index, sampling_locations, attn_weights)
+    _check(grad_output.is_cuda and grad_output.dtype in _FLOAT_CODES, "grad_output: float tensor on the GPU expected")
+    lib = _lib.load()
+    dt = value.dtype
+    value = value.contiguous()
+    shapes, lsi = spatial_shapes.int().contiguous(), level_start_index.int().contiguous()
+    loc, attn = sampling_locations.to(dt).contiguous(), attn_weights.to(dt).contiguous()
+    go = grad_output.to(dt).contiguous()
+    gv, ga = torch.empty_like(value), torch.empty_like(attn)
+    code = _FLOAT_CODES[dt]
+    nbytes = lib.mxd_gka_backward_workspace_bytes(code, *dims)
+    workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=value.device)
+    with torch.cuda.device(value.device):
+        rc = lib.mxd_gka_backward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(), attn.data_ptr(),
+                                  go.data_ptr(), gv.data_ptr(), ga.data_ptr(), workspace.data_ptr(), nbytes, code, *dims,
+                                  torch.cuda.current_stream().cuda_stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return gv, ga

@@ -22,12 +22,15 @@ from .ops.deformable_aggregation import (  # noqa: F401,E402
     deformable_aggregation,
     npu_deformable_aggregation,
 )
+from .ops.geometric_kernel_attention import GeometricKernelAttentionFunc, geometric_kernel_attention  # noqa: F401,E402
 from .ops.msda_fused import (  # noqa: F401,E402
     MultiScaleDeformableAttnFusedFunction,
     multi_scale_deformable_attn_fused,
 )
 
 __all__ = [
+    "GeometricKernelAttentionFunc",
+    "geometric_kernel_attention",
     "AdsDeformableAggregation",
     "deformable_aggregation",
     "npu_deformable_aggregation",

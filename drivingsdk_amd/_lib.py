@@ -25,6 +25,9 @@ EXPORTS = (
     "mxd_dagg_forward",
     "mxd_dagg_backward_workspace_bytes",
     "mxd_dagg_backward",
+    "mxd_gka_forward",
+    "mxd_gka_backward_workspace_bytes",
+    "mxd_gka_backward",
 )
 
 
@@ -78,6 +81,12 @@ def load():
     lib.mxd_dagg_backward_workspace_bytes.argtypes = [ci] + [i64] * 8
     lib.mxd_dagg_backward.restype = ci
     lib.mxd_dagg_backward.argtypes = [p] * 10 + [ctypes.c_size_t, ci] + [i64] * 8 + [p]
+    lib.mxd_gka_forward.restype = ci
+    lib.mxd_gka_forward.argtypes = [p] * 6 + [ci] + [i64] * 7 + [p]
+    lib.mxd_gka_backward_workspace_bytes.restype = ctypes.c_size_t
+    lib.mxd_gka_backward_workspace_bytes.argtypes = [ci] + [i64] * 7
+    lib.mxd_gka_backward.restype = ci
+    lib.mxd_gka_backward.argtypes = [p] * 9 + [ctypes.c_size_t, ci] + [i64] * 7 + [p]
     _lib = lib
     return lib
 

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             const int l = sr.l;
             const float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
             const bool inside = SRC != kSrcDagg || (cx > 0.0f && cx < 1.0f && cy > 0.0f && cy < 1.0f);
-            const Sample sm = sample_geometry(cx, cy, lvl[l], a.nk, inside);
+            const Sample sm = source_geometry<SRC>(cx, cy, lvl[l], a.nk, inside);
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
                 if ((sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0) {
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     l = sr.l;
                 }
                 const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active && inside);
+                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside);
                 Entry en;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     const float aw = to_f32(attn[sr.w_e]);
                     const int l = sr.l;
                     const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                    const Sample sm = sample_geometry(x, y, lvl[l], a.nk, inside);
+                    const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, inside);
                     const f32x4 dd = dots[u * kChunk + sl];
                     float ga = 0.f, gx = 0.f, gy = 0.f;
                     if (sm.valid) {
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                             unsafeAtomicAdd(part, gx);
                             unsafeAtomicAdd(part + 1, gy);
                         }
-                    } else {
+                    } else if constexpr (SRC != kSrcGka) {  // (pixel-index locations have no gradient)
                         gloc[2 * sr.loc_e] = from_f32<T>(gx);
                         gloc[2 * sr.loc_e + 1] = from_f32<T>(gy);
                     }
@@ -420,7 +420,12 @@ template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
 {
     const dim3 grid(a.plan.grid), block(a.plan.block);
-    if (a.cams > 0) {
+    if (a.gka) {
+        if (scatter)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcGka>), grid, block, a.plan.lds_bytes, stream, a);
+        else
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcGka>), grid, block, a.plan.lds_bytes, stream, a);
+    } else if (a.cams > 0) {
         if (scatter)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcDagg>), grid, block, a.plan.lds_bytes, stream, a);
         else

@@ -305,9 +305,10 @@ int mxd_msda_decode_block(const mxd_msda_plan* plan, uint32_t block_index, int64
     return 1;
 }
 
-int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
-                     const void* sampling_loc, const void* attn_weight, void* output, int dtype, int64_t bs, int64_t nk,
-                     int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np, void* hip_stream)
+static int forward_common(int gka, const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                          const void* sampling_loc, const void* attn_weight, void* output, int dtype, int64_t bs,
+                          int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
+                          void* hip_stream)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     int rc = check_dims(dtype, d);
@@ -327,9 +328,26 @@ int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int
     a.loc = sampling_loc;
     a.attn = attn_weight;
     a.out = output;
+    a.gka = gka;
     const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_forward: launch failed: %s", hipGetErrorString(e));
     return MXD_OK;
+}
+
+int mxd_msda_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                     const void* sampling_loc, const void* attn_weight, void* output, int dtype, int64_t bs, int64_t nk,
+                     int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np, void* hip_stream)
+{
+    return forward_common(0, value, spatial_shapes, level_start_index, sampling_loc, attn_weight, output, dtype, bs, nk,
+                          nh, hd, nl, nl_attn, nq, np, hip_stream);
+}
+
+int mxd_gka_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                    const void* sampling_locations, const void* attn_weights, void* output, int dtype, int64_t bs,
+                    int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nq, int64_t np, void* hip_stream)
+{
+    return forward_common(1, value, spatial_shapes, level_start_index, sampling_locations, attn_weights, output, dtype,
+                          bs, nk, nh, hd, nl, nl, nq, np, hip_stream);
 }
 
 int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
@@ -372,17 +390,17 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
     return bwd_layout(dtype, d).total;
 }
 
-int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
-                      const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
-                      void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype, int64_t bs,
-                      int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
-                      int flags, void* hip_stream)
+static int backward_common(int gka, const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                           const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
+                           void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype,
+                           int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq,
+                           int64_t np, int flags, void* hip_stream)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
     if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !grad_output || !grad_value ||
-        !grad_loc || !grad_attn)
+        (!grad_loc && !gka) || !grad_attn)
         return fail(MXD_E_NULL, "mxd_msda_backward: NULL data pointer");
     const BwdLayout L = bwd_layout(dtype, d);
     const size_t need = L.total;
@@ -418,6 +436,7 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     a.tbl_stride = (int32_t)L.tbl_stride;
     a.grad_loc = grad_loc;
     a.grad_attn = grad_attn;
+    a.gka = gka;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * nk * nh * hd;
     hipError_t e = hipSuccess;
@@ -439,6 +458,34 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: rounding launch failed: %s", hipGetErrorString(e));
     }
     return MXD_OK;
+}
+
+int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                      const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
+                      void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype, int64_t bs,
+                      int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
+                      int flags, void* hip_stream)
+{
+    return backward_common(0, value, spatial_shapes, level_start_index, sampling_loc, attn_weight, grad_output,
+                           grad_value, grad_loc, grad_attn, workspace, workspace_bytes, dtype, bs, nk, nh, hd, nl,
+                           nl_attn, nq, np, flags, hip_stream);
+}
+
+size_t mxd_gka_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
+                                        int64_t nq, int64_t np)
+{
+    return mxd_msda_backward_workspace_bytes(dtype, bs, nk, nh, hd, nl, nl, nq, np);
+}
+
+int mxd_gka_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                     const void* sampling_locations, const void* attn_weights, const void* grad_output,
+                     void* grad_value, void* grad_attn_weights, void* workspace, size_t workspace_bytes, int dtype,
+                     int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nq, int64_t np,
+                     void* hip_stream)
+{
+    return backward_common(1, value, spatial_shapes, level_start_index, sampling_locations, attn_weights, grad_output,
+                           grad_value, nullptr, grad_attn_weights, workspace, workspace_bytes, dtype, bs, nk, nh, hd, nl,
+                           nl, nq, np, 0, hip_stream);
 }
 
 int mxd_dagg_forward(const void* mc_ms_feat, const int32_t* spatial_shape, const int32_t* scale_start_index,

@@ -34,6 +34,7 @@ struct KArgs {
     int32_t cams;
     int32_t scales;
     uint32_t sc_magic;     // ceil(2^20/scales): level / scales
+    int32_t gka;           // geometric kernel attention: locations are pixel indices, one pixel per sample
     int32_t sc_pow2;       // scales is a power of two that divides 16: location gradients are summed over the
                            // scales across lanes and stored once; otherwise they are added with atomics
     const void* grad_out;  // backward only from here
@@ -61,7 +62,7 @@ struct KArgs {
 };
 
 // Where a kernel takes the location and the weight of sample s of unit (b, q, h) from.
-enum : int { kSrcPlain = 0, kSrcFused = 1, kSrcDagg = 2 };
+enum : int { kSrcPlain = 0, kSrcFused = 1, kSrcDagg = 2, kSrcGka = 3 };
 struct SampleRef {
     int64_t loc_e;  // index of the (x, y) pair
     int64_t w_e;    // index of the weight
@@ -274,6 +275,40 @@ __device__ inline Sample sample_geometry(float x, float y, i32x4 level, int32_t 
         s.w[k] = s.valid ? wt[k] : 0.0f;
     }
     return s;
+}
+
+// Geometric kernel attention (reference: mx_driving/ops/geometric_kernel_attention.py,
+// kernels/geometric_kernel_attention/op_kernel/geometric_kernel_attention.cpp:150-160): the location is a
+// pixel index pair (x, y), clamped to the level; the sample is that one pixel with weight 1, no interpolation.
+__device__ inline Sample gka_geometry(float x, float y, i32x4 level, int32_t nk, bool active)
+{
+    Sample s;
+    const int32_t H = level.x, W = level.y, base = level.z;
+    s.Wf = (float)W;
+    s.Hf = (float)H;
+    s.lw = s.lh = 0.0f;
+    s.valid = active && H > 0 && W > 0 && x == x && y == y;  // NaN locations contribute nothing
+    int32_t xi = s.valid ? (int32_t)__builtin_fminf(__builtin_fmaxf(x, -1.0f), 2147483520.0f) : 0;
+    int32_t yi = s.valid ? (int32_t)__builtin_fminf(__builtin_fmaxf(y, -1.0f), 2147483520.0f) : 0;
+    xi = xi < 0 ? 0 : (xi > W - 1 ? W - 1 : xi);
+    yi = yi < 0 ? 0 : (yi > H - 1 ? H - 1 : yi);
+    const int32_t p = base + yi * W + xi;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        s.pix[k] = p + k;  // corners 1..3 are never valid
+        s.cvalid[k] = false;
+        s.w[k] = 0.0f;
+    }
+    s.cvalid[0] = s.valid && ((uint32_t)p < (uint32_t)nk);
+    s.w[0] = s.valid ? 1.0f : 0.0f;
+    return s;
+}
+
+template <int SRC>
+__device__ inline Sample source_geometry(float x, float y, i32x4 level, int32_t nk, bool active)
+{
+    if constexpr (SRC == kSrcGka) return gka_geometry(x, y, level, nk, active);
+    else return sample_geometry(x, y, level, nk, active);
 }
 
 // ---- sum over the `lanes` (power of two <= 64) lanes that share a unit; every lane of the

@@ -145,7 +145,7 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
                 }
                 // deformable aggregation samples only strictly inside the image (0 < x, y < 1)
                 const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                const Sample sm = sample_geometry(x, y, lvl[l], a.nk, active && inside);
+                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside);
                 Entry en;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -194,7 +194,10 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
 template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, hipStream_t stream)
 {
-    if (a.cams > 0)
+    if (a.gka)
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcGka>), dim3(a.plan.grid), dim3(a.plan.block),
+                           a.plan.lds_bytes, stream, a);
+    else if (a.cams > 0)
         hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcDagg>), dim3(a.plan.grid), dim3(a.plan.block),
                            a.plan.lds_bytes, stream, a);
     else if (a.ref != nullptr)

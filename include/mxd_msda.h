@@ -188,6 +188,24 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
                       int64_t num_cams, int64_t num_scale, int64_t num_anchors, int64_t num_pts, int64_t num_groups,
                       void* hip_stream);
 
+/* ---- geometric kernel attention --------------------------------------------------------------
+ * Replaces geometric_kernel_attention_forward / _backward (mx_driving/csrc/GeometricKernelAttentionFunc.cpp:33-118)
+ * with the operator's own layouts: value [bs, nk, nh, hd] (the reference's binding permutes it itself),
+ * sampling_locations [bs, nq, nh, nl, np, 2] = (x, y) pixel indices in value's dtype (clamped to the level),
+ * attn_weights [bs, nq, nh, nl, np], output [bs, nq, nh*hd]:
+ *   output[b,q,h,:] = sum over (l, p) of attn * value[b, start_l + y*W_l + x, h, :].
+ * Gradients: grad_value and grad_attn_weights (locations are indices and have none). */
+int mxd_gka_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                    const void* sampling_locations, const void* attn_weights, void* output, int dtype, int64_t bs,
+                    int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nq, int64_t np, void* hip_stream);
+size_t mxd_gka_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
+                                        int64_t nq, int64_t np);
+int mxd_gka_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                     const void* sampling_locations, const void* attn_weights, const void* grad_output,
+                     void* grad_value, void* grad_attn_weights, void* workspace, size_t workspace_bytes, int dtype,
+                     int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nq, int64_t np,
+                     void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,8 +11,10 @@ from drivingsdk_amd.ops.deformable_aggregation import (  # noqa: F401,E402  (mx_
     deformable_aggregation,
     npu_deformable_aggregation,
 )
+from drivingsdk_amd.ops.geometric_kernel_attention import geometric_kernel_attention  # noqa: F401,E402
 
 __all__ = [
+    "geometric_kernel_attention",
     "deformable_aggregation",
     "npu_deformable_aggregation",
     "MultiScaleDeformableAttnFunction",

@@ -1,0 +1,69 @@
+"""Geometric kernel attention on the GPU against the CPU oracle.  Shapes after the reference's test
+(tests/torch/test_geometric_kernel_attention.py:118-124, batch sizes shrunk; its location recipe :22-33)."""
+import numpy as np
+import pytest
+import torch
+
+import mx_driving
+from drivingsdk_amd import _lib
+from oracle import gka_oracle as gka
+from util import BWD_FP32, FWD_FP32, HALF, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def make_inputs(shape, hw, seed=0):
+    bs, nq, hd, nh, nl, npts = shape
+    g = torch.Generator().manual_seed(seed)
+    sh = torch.tensor([list(hw)] * nl)
+    lsi = torch.cat((sh.new_zeros((1,)), sh.prod(1).cumsum(0)[:-1]))
+    nk = int(sh.prod(1).sum())
+    loc = torch.rand(bs, nq, nh, nl, npts, 2, generator=g)
+    loc[..., 0] = loc[..., 0] * (hw[1] + 6) - 3
+    loc[..., 1] = loc[..., 1] * (hw[0] + 6) - 3
+    loc = loc.long().float()                                   # as the reference test: truncated, passed as float
+    value = torch.rand(bs, nk, nh, hd, generator=g) * 3
+    attn = torch.rand(bs, nq, nh, nl, npts, generator=g)
+    go = torch.rand(bs, nq, nh * hd, generator=g) * 10
+    return value, sh, lsi, loc, attn, go
+
+
+def run_gpu(value, sh, lsi, loc, attn, go, device, dtype=torch.float32, loc_dtype=None):
+    v = value.to(device, dtype).requires_grad_()
+    a = attn.to(device, dtype).requires_grad_()
+    lo = loc.to(device, loc_dtype or dtype)
+    out = mx_driving.geometric_kernel_attention(v, sh.to(device), lsi.to(device), lo, a)
+    out.backward(go.to(device, dtype))
+    return [t.detach().double().cpu().numpy() for t in (out, v.grad, a.grad)]
+
+
+@pytest.mark.parametrize("shape,hw", [([3, 7156, 64, 4, 1, 15], (15, 25)), ([6, 1146, 64, 4, 1, 15], (6, 10)),
+                                      ([2, 4, 16, 4, 2, 15], (6, 10)), ([2, 333, 32, 8, 3, 4], (20, 30))])
+def test_reference_test_shapes(gpu_device, shape, hw):
+    inp = make_inputs(shape, hw, seed=shape[1])
+    want = (gka.forward(*inp[:5]),) + gka.backward(*inp)
+    got = run_gpu(*inp, gpu_device)
+    for name, g_, w_, tol in zip(("output", "grad_value", "grad_attn_weights"), got, want, (FWD_FP32, BWD_FP32, BWD_FP32)):
+        assert rel_err(g_, w_) <= tol, (name, rel_err(g_, w_))
+
+
+def test_integer_locations_and_float16(gpu_device):
+    inp = make_inputs([2, 100, 32, 4, 2, 6], (9, 13), seed=5)
+    want = gka.forward(*inp[:5])
+    got = run_gpu(*inp, gpu_device, loc_dtype=torch.int64)
+    assert rel_err(got[0], want) <= FWD_FP32
+    value, sh, lsi, loc, attn, go = inp
+    want16 = gka.forward(value.half().double(), sh, lsi, loc, attn.half().double())
+    got16 = run_gpu(*inp, gpu_device, dtype=torch.float16)
+    assert rel_err(got16[0], want16) <= HALF
+
+
+def test_error_paths(gpu_device):
+    value, sh, lsi, loc, attn, go = [t.to(gpu_device) if isinstance(t, torch.Tensor) else t
+                                     for t in make_inputs([1, 5, 16, 2, 1, 3], (4, 4))]
+    with pytest.raises(RuntimeError, match="sampling_locations: float16, float32, int32 or int64"):
+        mx_driving.geometric_kernel_attention(value, sh, lsi, loc.double(), attn)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        mx_driving.geometric_kernel_attention(value.cpu(), sh.cpu(), lsi.cpu(), loc.cpu(), attn.cpu())
+    lib = _lib.load()
+    assert lib.mxd_gka_forward(None, None, None, None, None, None, 0, 1, 16, 2, 16, 1, 5, 3, None) == -3
