@@ -129,3 +129,15 @@ def test_error_paths(gpu_device):
     assert lib.mxd_dagg_forward(None, None, None, None, None, None, 0, 1, 64, 32, 1, 1, 4, 3, 8, None) == -3
     assert lib.mxd_dagg_forward(None, None, None, None, None, None, 0, 1, 64, 30, 1, 1, 4, 3, 8, None) == -2
     assert lib.mxd_dagg_backward_workspace_bytes(0, 1, 64, 32, 1, 1, 4, 3, 8) > 0
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_small_problems(gpu_device, seed):
+    rng = np.random.default_rng(500 + seed)
+    cams, scales = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+    G = int(rng.choice([1, 2, 3, 4, 8]))
+    C = G * int(rng.choice([1, 2, 4, 5, 8, 16, 32, 40]))
+    maps = [[(int(rng.integers(1, 40)), int(rng.integers(1, 40))) for _ in range(scales)] for _ in range(cams)]
+    bs, A, P = int(rng.integers(1, 4)), int(rng.integers(1, 200)), int(rng.integers(1, 14))
+    print("case", bs, C, G, A, P, maps, flush=True)
+    check(make_inputs(bs, C, G, A, P, maps, seed=seed, pad=True), gpu_device)

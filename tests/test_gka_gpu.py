@@ -67,3 +67,17 @@ def test_error_paths(gpu_device):
         mx_driving.geometric_kernel_attention(value.cpu(), sh.cpu(), lsi.cpu(), loc.cpu(), attn.cpu())
     lib = _lib.load()
     assert lib.mxd_gka_forward(None, None, None, None, None, None, 0, 1, 16, 2, 16, 1, 5, 3, None) == -3
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_small_problems(gpu_device, seed):
+    rng = np.random.default_rng(700 + seed)
+    shape = [int(rng.integers(1, 4)), int(rng.integers(1, 500)), int(rng.choice([1, 3, 8, 16, 32, 64, 100])),
+             int(rng.integers(1, 9)), int(rng.integers(1, 4)), int(rng.integers(1, 17))]
+    hw = (int(rng.integers(1, 30)), int(rng.integers(1, 30)))
+    print("case", shape, hw, flush=True)
+    inp = make_inputs(shape, hw, seed=seed)
+    want = (gka.forward(*inp[:5]),) + gka.backward(*inp)
+    got = run_gpu(*inp, gpu_device)
+    for g_, w_, tol in zip(got, want, (FWD_FP32, BWD_FP32, BWD_FP32)):
+        assert rel_err(g_, w_) <= tol

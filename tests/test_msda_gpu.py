@@ -377,3 +377,27 @@ def test_backward_launch_variants_agree_with_the_oracle(gpu_device, monkeypatch,
         inp = workloads.make_inputs(name, with_grad_output=True, scale_queries=scale)
         errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
         print(env, name, errs)
+
+
+def _random_case(seed):
+    """A random small problem: odd sizes everywhere, locations reaching outside the image."""
+    rng = np.random.default_rng(seed)
+    bs, nq, nh = int(rng.integers(1, 4)), int(rng.integers(1, 700)), int(rng.integers(1, 10))
+    hd = int(rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 64, 96, 128, 256]))
+    nl, npts = int(rng.integers(1, 6)), int(rng.integers(1, 10))
+    levels = [(int(rng.integers(1, 48)), int(rng.integers(1, 48))) for _ in range(nl)]
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    g = torch.Generator().manual_seed(seed)
+    value = torch.randn(bs, nk, nh, hd, generator=g)
+    loc = torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.3 - 0.15
+    attn = torch.rand(bs, nq, nh, nl, npts, generator=g)
+    grad_out = torch.randn(bs, nq, nh * hd, generator=g)
+    return workloads.MsdaInputs(value, shapes, lsi, loc, attn, grad_out), (bs, nq, nh, hd, levels, npts)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_small_problems(gpu_device, seed):
+    inp, desc = _random_case(1000 + seed)
+    print("case", desc, flush=True)
+    _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
