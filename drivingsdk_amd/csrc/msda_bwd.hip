@@ -26,6 +26,8 @@
 // the counts into run starts inside its own slab of the record array, publishes them as its
 // row of the run table, and then -- where it computes grad_loc anyway -- drops every record
 // at the next free position of its tile's run (one LDS integer atomic per record).
+#include <type_traits>
+
 #include "msda_device.h"
 
 namespace mxd {
@@ -202,26 +204,39 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             // ---- gather and dots -------------------------------------------------------
             const int ns = (a.S - c0) < kChunk ? (a.S - c0) : kChunk;
             const Entry* mine = stage + g * kChunkStride;
-            for (int sl = 0; sl < ns; ++sl) {
-                const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
-                float d[4] = {0.f, 0.f, 0.f, 0.f};
+            // (the reduction width is a compile-time constant inside the loop: with a run-time width its
+            // uniform branches keep the row loads of the next samples from being issued early)
+            auto gather_dots = [&](auto lg) {
+                constexpr int LG = decltype(lg)::value;
+#pragma unroll 2
+                for (int sl = 0; sl < ns; ++sl) {
+                    const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
+                    float d[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int p = 0; p < NPASS; ++p) {
-                    typename RowIO<T, VEC>::raw_t raw[4];
+                    for (int p = 0; p < NPASS; ++p) {
+                        typename RowIO<T, VEC>::raw_t raw[4];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
+                        for (int k = 0; k < 4; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        float v[VEC];
-                        RowIO<T, VEC>::unpack(raw[k], v);
+                        for (int k = 0; k < 4; ++k) {
+                            float v[VEC];
+                            RowIO<T, VEC>::unpack(raw[k], v);
 #pragma unroll
-                        for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
+                            for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
+                        }
                     }
-                }
-                f32x4 dsum;
+                    f32x4 dsum;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) dsum[k] = group_sum(d[k], lpr_log2);
-                if (c == 0) dots[g * kChunk + sl] = dsum;
+                    for (int k = 0; k < 4; ++k) dsum[k] = group_sum<LG>(d[k]);
+                    if (c == 0) dots[g * kChunk + sl] = dsum;
+                }
+            };
+            switch (lpr_log2) {
+                case 2: gather_dots(std::integral_constant<int, 2>{}); break;
+                case 3: gather_dots(std::integral_constant<int, 3>{}); break;
+                case 4: gather_dots(std::integral_constant<int, 4>{}); break;
+                case 5: gather_dots(std::integral_constant<int, 5>{}); break;
+                default: gather_dots(std::integral_constant<int, 6>{}); break;
             }
             wave_lds_sync();
             // ---- scatter: grad_value[row_c] += (w_c*attn) * grad_out row --------------------

@@ -319,15 +319,16 @@ __device__ inline float dpp_xchg(float v)
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
 }
 
-__device__ inline float group_sum(float v, int lanes_log2)
+template <int LANES_LOG2>
+__device__ inline float group_sum(float v)
 {
     // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror
-    if (lanes_log2 >= 1) v += dpp_xchg<0xB1>(v);
-    if (lanes_log2 >= 2) v += dpp_xchg<0x4E>(v);
-    if (lanes_log2 >= 3) v += dpp_xchg<0x141>(v);
-    if (lanes_log2 >= 4) v += dpp_xchg<0x140>(v);
-    if (lanes_log2 >= 5) v += __shfl_xor(v, 16, 64);
-    if (lanes_log2 >= 6) v += __shfl_xor(v, 32, 64);
+    if constexpr (LANES_LOG2 >= 1) v += dpp_xchg<0xB1>(v);
+    if constexpr (LANES_LOG2 >= 2) v += dpp_xchg<0x4E>(v);
+    if constexpr (LANES_LOG2 >= 3) v += dpp_xchg<0x141>(v);
+    if constexpr (LANES_LOG2 >= 4) v += dpp_xchg<0x140>(v);
+    if constexpr (LANES_LOG2 >= 5) v += __shfl_xor(v, 16, 64);
+    if constexpr (LANES_LOG2 >= 6) v += __shfl_xor(v, 32, 64);
     return v;
 }
 
