@@ -1,7 +1,7 @@
 // Backward kernel of multi-scale deformable attention for gfx950 (MI355X), wave64.
 //
 // For every sample (b,q,h,l,p) with g = grad_out[b,q,h,:]:
-//   grad_value[row_c] += w_c * attn * g                  (4 corner rows, fp32 atomics)
+//   grad_value[row_c] += w_c * attn * g                  (4 corner rows; left to the tile pass, or fp32 atomics)
 //   d_c = dot(value[row_c], g)
 //   grad_attn = sum_c w_c d_c
 //   grad_x = W attn (hh (d2-d1) + lh (d4-d3)),  grad_y = H attn (hw (d3-d1) + lw (d4-d2))
@@ -13,8 +13,8 @@
 //   * per staged sample the lanes of a unit fetch the 4 corner rows with one buffer load
 //     each and form partial dots with the register-resident grad_out row; the partial dots
 //     are summed across the unit's lanes with DPP and parked in LDS;
-//   * the scatter then walks the staged samples again with a row-contiguous lane layout and
-//     issues buffer atomics (out-of-image corners carry an out-of-range offset: the load
+//   * (SCATTER = true only) the scatter then walks the staged samples again with a row-contiguous lane
+//     layout and issues buffer atomics (out-of-image corners carry an out-of-range offset: the load
 //     yields 0, the atomic is dropped by the hardware range check);
 //   * the geometry lanes turn the reduced dots into grad_attn / grad_loc and store them
 //     coalesced.

@@ -1,5 +1,7 @@
 // C ABI entry points (include/mxd_msda.h): argument checks, launch geometry, enqueue.
-// Host code only; the kernels live in msda_fwd.hip / msda_bwd.hip.
+// Host code only; the kernels live in msda_fwd.hip, msda_bwd.hip and msda_bwd_tiles.hip.  Multi-scale
+// deformable attention, its fused form, deformable aggregation and geometric kernel attention are the same
+// three kernels with different sample sources (msda_device.h: sample_ref, source_geometry).
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
@@ -314,7 +316,7 @@ static int forward_common(int gka, const void* value, const int32_t* spatial_sha
     int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
     if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !output)
-        return fail(MXD_E_NULL, "mxd_msda_forward: NULL data pointer");
+        return fail(MXD_E_NULL, "%s: NULL data pointer", gka ? "mxd_gka_forward" : "mxd_msda_forward");
     int align = ptr_align(value);
     if (ptr_align(output) < align) align = ptr_align(output);
     mxd::KArgs a;
@@ -330,7 +332,7 @@ static int forward_common(int gka, const void* value, const int32_t* spatial_sha
     a.out = output;
     a.gka = gka;
     const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
-    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_forward: launch failed: %s", hipGetErrorString(e));
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", gka ? "mxd_gka_forward" : "mxd_msda_forward", hipGetErrorString(e));
     return MXD_OK;
 }
 
@@ -397,24 +399,25 @@ static int backward_common(int gka, const void* value, const int32_t* spatial_sh
                            int64_t np, int flags, void* hip_stream)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
+    const char* who = gka ? "mxd_gka_backward" : "mxd_msda_backward";
     int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
     if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !grad_output || !grad_value ||
         (!grad_loc && !gka) || !grad_attn)
-        return fail(MXD_E_NULL, "mxd_msda_backward: NULL data pointer");
+        return fail(MXD_E_NULL, "%s: NULL data pointer", who);
     const BwdLayout L = bwd_layout(dtype, d);
     const size_t need = L.total;
     if (need > 0 && (!workspace || workspace_bytes < need))
-        return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace of %zu bytes required, %zu given", need,
+        return fail(MXD_E_WORKSPACE, "%s: workspace of %zu bytes required, %zu given", who, need,
                     workspace ? workspace_bytes : (size_t)0);
     if (need > 0 && (reinterpret_cast<uintptr_t>(workspace) & 15u))
-        return fail(MXD_E_WORKSPACE, "mxd_msda_backward: workspace must be 16-byte aligned");
+        return fail(MXD_E_WORKSPACE, "%s: workspace must be 16-byte aligned", who);
     const bool half = elem_size(dtype) == 2;
     if ((flags & MXD_BWD_ACCUMULATE) && half)
-        return fail(MXD_E_DTYPE, "mxd_msda_backward: MXD_BWD_ACCUMULATE is only available for float32");
+        return fail(MXD_E_DTYPE, "%s: MXD_BWD_ACCUMULATE is only available for float32", who);
     char* ws = static_cast<char*>(workspace);
     float* image = half ? reinterpret_cast<float*>(ws + L.tbl_bytes + L.rec_bytes) : static_cast<float*>(grad_value);
-    if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_msda_backward: grad_value is not 4-byte aligned");
+    if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "%s: grad_value is not 4-byte aligned", who);
     int align = ptr_align(value);
     if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
     mxd::KArgs a;
@@ -441,21 +444,21 @@ static int backward_common(int gka, const void* value, const int32_t* spatial_sh
     const size_t n = (size_t)bs * nk * nh * hd;
     hipError_t e = hipSuccess;
     if (!(flags & MXD_BWD_ACCUMULATE)) e = mxd::launch_fill_zero(image, n, stream);
-    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: zero-fill launch failed: %s", hipGetErrorString(e));
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: zero-fill launch failed: %s", who, hipGetErrorString(e));
     const bool atomic_mode = !L.tiles;
     e = mxd::launch_backward(dtype, a, atomic_mode, stream);
-    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: launch failed: %s", hipGetErrorString(e));
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(e));
     if (!atomic_mode) {
         mxd::TileArgs t;
         rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
         if (rc != MXD_OK) return rc;
         t.store_vec = (hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
         e = mxd::launch_gradv_tiles(dtype, a, t, stream);
-        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: tile kernel launch failed: %s", hipGetErrorString(e));
+        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: tile kernel launch failed: %s", who, hipGetErrorString(e));
     }
     if (half) {
         e = mxd::launch_round(dtype, image, grad_value, n, stream);
-        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_backward: rounding launch failed: %s", hipGetErrorString(e));
+        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: rounding launch failed: %s", who, hipGetErrorString(e));
     }
     return MXD_OK;
 }
