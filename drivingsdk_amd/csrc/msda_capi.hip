@@ -179,7 +179,15 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
     return MXD_OK;
 }
 
-int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_plan* p)
+// Bytes of LDS the plain forward sets aside for the rows of the last levels (0: none).  Needs 16-byte lanes.
+int forward_cache_bytes(int vec, int es)
+{
+    const int v = env_int("MXD_MSDA_FWD_LDS", 32768);
+    return (vec * es == 16 && v >= 1024 && v <= 65536) ? (v & ~15) : 0;
+}
+
+// level_cache: in/out, bytes of LDS for the forward's level cache (asked for -> granted)
+int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_plan* p, int* level_cache = nullptr)
 {
     const int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
@@ -203,6 +211,22 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     const BwdLayout L = bwd_layout(dtype, d);
     // the tile pass wants L.tile_q queries per workgroup of the first backward kernel
     if (backward) iters = L.tiles ? (int)(L.tile_q / (p->units_per_wave * p->waves_per_block)) : 1;
+    int cache = (level_cache && *level_cache && !backward) ? forward_cache_bytes(vec, es) : 0;
+    if (cache > 0) {
+        // 8 wavefronts share one copy of the cached rows and work through 256 queries; two such workgroups
+        // must fit a CU (80 KiB each), else fewer wavefronts, else no cache
+        int waves = 8;
+        while (waves > 2 && mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)waves * p->units_per_wave *
+                                    (mxd::kChunkStride * sizeof(mxd::Entry) + 2 * sizeof(float)) + cache > 80 * 1024)
+            waves >>= 1;
+        if (waves > 2) {
+            p->waves_per_block = waves;
+            iters = 256 / (p->units_per_wave * p->waves_per_block);
+            if (iters < 1) iters = 1;
+        } else {
+            cache = 0;
+        }
+    }
     p->iters = iters;
     p->tile_q = p->units_per_wave * p->waves_per_block * p->iters;
     const int64_t ntiles = (d.nq + p->tile_q - 1) / p->tile_q;
@@ -216,6 +240,8 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     p->lds_bytes = (uint32_t)(mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)p->waves_per_block * p->units_per_wave * per_unit);
     if (backward && L.tiles) p->lds_bytes += (uint32_t)((mxd::kMaxLevels + L.tbl_stride) * sizeof(int32_t));
     if (!backward) p->lds_bytes += (uint32_t)(p->waves_per_block * p->units_per_wave * 2 * sizeof(float));  // softmax statistics (fused form)
+    if (cache > 0) p->lds_bytes += (uint32_t)cache;
+    if (level_cache) *level_cache = cache;
     return MXD_OK;
 }
 
@@ -291,7 +317,8 @@ int mxd_msda_make_plan(int backward, int dtype, int64_t bs, int64_t nk, int64_t 
 {
     if (!plan) return fail(MXD_E_NULL, "plan is NULL");
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
-    return make_plan(backward != 0, dtype, d, align_bytes, plan);
+    int cache = 1;
+    return make_plan(backward != 0, dtype, d, align_bytes, plan, &cache);
 }
 
 int mxd_msda_decode_block(const mxd_msda_plan* plan, uint32_t block_index, int64_t bs, int64_t nh, int64_t nq,
@@ -321,7 +348,8 @@ static int forward_common(int gka, const void* value, const int32_t* spatial_sha
     if (ptr_align(output) < align) align = ptr_align(output);
     mxd::KArgs a;
     memset(&a, 0, sizeof(a));
-    rc = make_plan(0, dtype, d, align, &a.plan);
+    int cache = gka == 0;
+    rc = make_plan(0, dtype, d, align, &a.plan, &cache);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
     a.value = value;
@@ -331,6 +359,7 @@ static int forward_common(int gka, const void* value, const int32_t* spatial_sha
     a.attn = attn_weight;
     a.out = output;
     a.gka = gka;
+    a.lds_cache_bytes = cache;
     const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", gka ? "mxd_gka_forward" : "mxd_msda_forward", hipGetErrorString(e));
     return MXD_OK;

@@ -34,6 +34,7 @@ struct KArgs {
     int32_t cams;
     int32_t scales;
     uint32_t sc_magic;     // ceil(2^20/scales): level / scales
+    int32_t lds_cache_bytes;  // forward: LDS set aside for the rows of the last (coarsest) levels, 0 = none
     int32_t gka;           // geometric kernel attention: locations are pixel indices, one pixel per sample
     int32_t sc_pow2;       // scales is a power of two that divides 16: location gradients are summed over the
                            // scales across lanes and stored once; otherwise they are added with atomics

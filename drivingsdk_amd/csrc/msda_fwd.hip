@@ -35,10 +35,11 @@
 
 namespace mxd {
 
-template <typename T, int VEC, int NPASS, int SRC>
-__global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
+template <typename T, int VEC, int NPASS, int SRC, bool LDSC>
+__global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs a)
 {
     constexpr bool FUSED = SRC == kSrcFused;
+    static_assert(!LDSC || (SRC == kSrcPlain && VEC * sizeof(T) == 16), "the level cache is built for 16-byte lanes");
     extern __shared__ __align__(16) unsigned char smem[];
     i32x4* lvl = reinterpret_cast<i32x4*>(smem);                               // [kMaxLevels]
     Entry* stage_all = reinterpret_cast<Entry*>(smem + kMaxLevels * sizeof(i32x4));
@@ -55,6 +56,46 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
         lvl[i] = L;
     }
     __syncthreads();
+
+    // ---- level cache (LDSC): the rows of this (batch, head) for the last levels, as many as fit ----------
+    // The gather is bound by the vector-memory pipeline (64 bytes per clock per CU); rows held in LDS are read
+    // through the LDS pipeline instead, in parallel with it.  Levels are cached from the last one backwards
+    // while level_start_index is ascending and the rows from that level's start to the end of value fit.
+    __shared__ int32_t c_first_s, c_base_s, c_rows_s;
+    unsigned char* cache = smem + kMaxLevels * sizeof(i32x4) +
+                           (size_t)a.plan.waves_per_block * a.plan.units_per_wave * (kChunkStride * sizeof(Entry) + 2 * sizeof(float));
+    const uint32_t row_bytes = (uint32_t)a.hd * sizeof(T);
+    int c_first = a.nl, c_base = 0, c_rows = 0;
+    if constexpr (LDSC) {
+        if (threadIdx.x == 0) {
+            int first = a.nl, base = 0;
+            const int cap_rows = (int)(a.lds_cache_bytes / row_bytes) - 1;  // one more row of zeros
+            for (int l = a.nl - 1; l >= 0; --l) {
+                const int b0 = lvl[l].z;
+                if (b0 < 0 || b0 >= a.nk || a.nk - b0 > cap_rows || (l < a.nl - 1 && b0 > lvl[l + 1].z)) break;
+                first = l;
+                base = b0;
+            }
+            c_first_s = first;
+            c_base_s = base;
+            c_rows_s = first < a.nl ? a.nk - base : 0;
+        }
+        __syncthreads();
+        c_first = c_first_s;
+        c_base = c_base_s;
+        c_rows = c_rows_s;
+        const int pieces = (int)(row_bytes / 16);
+        const char* src = static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes +
+                          (size_t)c_base * a.pitch_bytes + (size_t)wk.h * row_bytes;
+        for (int i = threadIdx.x; i < c_rows * pieces; i += blockDim.x) {
+            const int row = i / pieces, piece = i - row * pieces;
+            *reinterpret_cast<u32x4*>(cache + (size_t)row * row_bytes + piece * 16) =
+                *reinterpret_cast<const u32x4*>(src + (size_t)row * a.pitch_bytes + piece * 16);
+        }
+        for (int i = threadIdx.x; i < pieces; i += blockDim.x)
+            *reinterpret_cast<u32x4*>(cache + (size_t)c_rows * row_bytes + i * 16) = u32x4{0u, 0u, 0u, 0u};
+        __syncthreads();
+    }
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -84,6 +125,10 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
         chan_ok[p] = ch < a.hd;
         choff[p] = head_off + (chan_ok[p] ? ch * (uint32_t)sizeof(T) : 0u);
     }
+    // same lane offsets inside a cached row
+    uint32_t lds_choff[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) lds_choff[p] = choff[p] - head_off;
 
     const int entries = U * kChunk;  // staged samples per pass
     for (int it = 0; it < a.plan.iters; ++it) {
@@ -151,6 +196,12 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
                 for (int k = 0; k < 4; ++k) {
                     en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
                     en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
+                    if constexpr (LDSC) {
+                        // cached level: byte offset of the row in the cache; the row of zeros for a corner
+                        // outside the image
+                        if (l >= c_first)
+                            en.off[k] = (uint32_t)(sm.cvalid[k] ? sm.pix[k] - c_base : c_rows) * row_bytes;
+                    }
                 }
                 stage[u * kChunkStride + sl] = en;
             }
@@ -159,8 +210,14 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
             // ---- gather + weighted sum ----------------------------------------------------
             const int ns = (a.S - c0) < kChunk ? (a.S - c0) : kChunk;
             const Entry* mine = stage + g * kChunkStride;
+            // samples are level-major: those of the cached levels are the tail of the unit's list
+            int n_mem = ns;
+            if constexpr (LDSC) {
+                n_mem = c_first * a.np - c0;
+                n_mem = n_mem < 0 ? 0 : (n_mem > ns ? ns : n_mem);
+            }
 #pragma unroll 4
-            for (int sl = 0; sl < ns; ++sl) {
+            for (int sl = 0; sl < n_mem; ++sl) {
                 const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
                 const f32x4 w = *reinterpret_cast<const f32x4*>(mine[sl].w);
 #pragma unroll
@@ -174,6 +231,27 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
                         RowIO<T, VEC>::unpack(raw[k], v);
 #pragma unroll
                         for (int e = 0; e < VEC; ++e) acc[p][e] = __builtin_fmaf(w[k], v[e], acc[p][e]);
+                    }
+                }
+            }
+            if constexpr (LDSC) {
+#pragma unroll 4
+                for (int sl = n_mem; sl < ns; ++sl) {
+                    const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
+                    const f32x4 w = *reinterpret_cast<const f32x4*>(mine[sl].w);
+#pragma unroll
+                    for (int p = 0; p < NPASS; ++p) {
+                        typename RowIO<T, VEC>::raw_t raw[4];
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            raw[k] = *reinterpret_cast<const typename RowIO<T, VEC>::raw_t*>(cache + off[k] + lds_choff[p]);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            float v[VEC];
+                            RowIO<T, VEC>::unpack(raw[k], v);
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) acc[p][e] = __builtin_fmaf(w[k], v[e], acc[p][e]);
+                        }
                     }
                 }
             }
@@ -194,18 +272,30 @@ __global__ __launch_bounds__(256) void msda_fwd_kernel(const KArgs a)
 template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, hipStream_t stream)
 {
+    const dim3 grid(a.plan.grid), block(a.plan.block);
     if (a.gka)
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcGka>), dim3(a.plan.grid), dim3(a.plan.block),
-                           a.plan.lds_bytes, stream, a);
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcGka, false>), grid, block, a.plan.lds_bytes, stream, a);
     else if (a.cams > 0)
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcDagg>), dim3(a.plan.grid), dim3(a.plan.block),
-                           a.plan.lds_bytes, stream, a);
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcDagg, false>), grid, block, a.plan.lds_bytes, stream, a);
     else if (a.ref != nullptr)
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcFused>), dim3(a.plan.grid), dim3(a.plan.block),
-                           a.plan.lds_bytes, stream, a);
-    else
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain>), dim3(a.plan.grid), dim3(a.plan.block),
-                           a.plan.lds_bytes, stream, a);
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcFused, false>), grid, block, a.plan.lds_bytes, stream, a);
+    else if (a.lds_cache_bytes > 0) {
+        if constexpr (VEC * sizeof(T) == 16) {
+            // more than the 64 KiB of dynamic LDS a kernel gets by default: opt in once per instantiation
+            static bool raised = false;
+            if (!raised) {
+                const hipError_t e = hipFuncSetAttribute(
+                    reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true>),
+                    hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+                if (e != hipSuccess) return e;
+                raised = true;
+            }
+            hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true>), grid, block, a.plan.lds_bytes, stream, a);
+        } else {
+            return hipErrorInvalidConfiguration;
+        }
+    } else
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, false>), grid, block, a.plan.lds_bytes, stream, a);
     return hipGetLastError();
 }
 

@@ -56,7 +56,7 @@ def test_plan_covers_every_unit_exactly_once(backward, dims):
         assert hd % plan.vec == 0
         assert plan.block == 64 * plan.waves_per_block
         assert plan.tile_q == plan.units_per_wave * plan.waves_per_block * plan.iters
-        assert plan.lds_bytes <= 64 * 1024
+        assert plan.lds_bytes <= 80 * 1024   # two workgroups per CU
         seen = {}
         work = (ctypes.c_int32 * 4)()
         for bid in range(plan.grid):
