@@ -310,3 +310,66 @@ def geometric_kernel_attention_backward(value, spatial_shapes, level_start_index
                                   torch.cuda.current_stream().cuda_stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return gv, ga
+
+
+# ---- 2-D grid sampler (mx_driving/csrc/GridSampler2dV2.cpp:33-99 of the reference) ------------------------------
+
+def grid_sampler2d_v2(input, grid, interpolation_mode, padding_mode, align_corners):
+    """input [N, C, H, W], grid [N, H_out, W_out, 2] -> output [N, C, H_out, W_out] (bilinear).  As in the reference's
+    binding the kernel works on channel-last data: input is permuted to NHWC before and the output back after."""
+    _check(input.layout == torch.strided and grid.layout == torch.strided,
+           "grid_sampler2d_v2(): expected input and grid to have torch.strided layout")
+    _check(input.dtype in _FLOAT_CODES and grid.dtype == input.dtype,
+           f"grid_sampler2d_v2(): float tensors of one dtype expected, but got input tensor with dtype: {input.dtype} "
+           f"and grid tensor with dtype: {grid.dtype}")
+    _check(input.dim() == 4 and grid.dim() == 4,
+           f"grid_sampler2d_v2(): input and grid must be 4D tensor, but got input with sizes {tuple(input.shape)} "
+           f"and grid with sizes {tuple(grid.shape)}")
+    _check(input.size(0) == grid.size(0),
+           f"grid_sampler2d_v2(): input and grid must have same batch size, but got input with sizes "
+           f"{tuple(input.shape)} and grid with sizes {tuple(grid.shape)}")
+    _check(grid.size(-1) == 2,
+           f"grid_sampler2d_v2(): grid must have size 2 in last dimension, but got grid with sizes {tuple(grid.shape)}")
+    _check(input.is_cuda and grid.is_cuda and input.device == grid.device,
+           "grid_sampler2d_v2(): input and grid must live on one GPU (this build has no CPU implementation)")
+    n, c, h_in, w_in = input.shape
+    _, h_out, w_out, _ = grid.shape
+    lib = _lib.load()
+    dt = input.dtype
+    x = input.permute(0, 2, 3, 1).contiguous()
+    g = grid.contiguous()
+    out = torch.empty((n, h_out, w_out, c), dtype=dt, device=input.device)
+    with torch.cuda.device(input.device):
+        rc = lib.mxd_grid_sampler2d_forward(x.data_ptr(), g.data_ptr(), out.data_ptr(), _FLOAT_CODES[dt], n, c, h_in,
+                                            w_in, h_out, w_out, int(interpolation_mode), int(padding_mode),
+                                            int(bool(align_corners)), torch.cuda.current_stream().cuda_stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return out.permute(0, 3, 1, 2).contiguous()
+
+
+def grid_sampler2d_v2_backward(grad_output, input_x, input_grid, interpolation_mode, padding_mode, align_corners):
+    """grad_output and input_x channel-last ([N, H_out, W_out, C], [N, H, W, C]) as the reference's binding takes
+    them (mx_driving/ops/grid_sampler2d_v2.py:64-70).  Returns (grad_x as an NCHW view, grad_grid)."""
+    _check(grad_output.dim() == 4, f"grad_output must to be a 4D Tensor, but got: {grad_output.dim()}")
+    _check(input_x.dim() == 4, f"input_x has to be a 4D Tensor, but got: {input_x.dim()}")
+    _check(input_grid.dim() == 4, f"input_grid has to be a 4D Tensor, but got: {input_grid.dim()}")
+    _check(all(t.is_cuda for t in (grad_output, input_x, input_grid)),
+           "grid_sampler2d_v2_backward(): all tensors must live on a GPU (this build has no CPU implementation)")
+    n, h_in, w_in, c = input_x.shape
+    _, h_out, w_out, _ = input_grid.shape
+    _check(tuple(grad_output.shape) == (n, h_out, w_out, c), "grad_output: expected [N, H_out, W_out, C]")
+    lib = _lib.load()
+    dt = input_x.dtype
+    _check(dt in _FLOAT_CODES, f"input_x: float tensor expected but got {dt}")
+    x, g, go = input_x.contiguous(), input_grid.to(dt).contiguous(), grad_output.to(dt).contiguous()
+    grad_x, grad_grid = torch.empty_like(x), torch.empty_like(g)
+    code = _FLOAT_CODES[dt]
+    nbytes = lib.mxd_grid_sampler2d_backward_workspace_bytes(code, n, c, h_in, w_in, h_out, w_out)
+    workspace = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.mxd_grid_sampler2d_backward(go.data_ptr(), x.data_ptr(), g.data_ptr(), grad_x.data_ptr(),
+                                             grad_grid.data_ptr(), workspace.data_ptr(), nbytes, code, n, c, h_in,
+                                             w_in, h_out, w_out, int(interpolation_mode), int(padding_mode),
+                                             int(bool(align_corners)), torch.cuda.current_stream().cuda_stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return grad_x.permute(0, 3, 1, 2), grad_grid

@@ -23,12 +23,15 @@ from .ops.deformable_aggregation import (  # noqa: F401,E402
     npu_deformable_aggregation,
 )
 from .ops.geometric_kernel_attention import GeometricKernelAttentionFunc, geometric_kernel_attention  # noqa: F401,E402
+from .ops.grid_sampler2d_v2 import GridSampler2dV2Function, grid_sampler2d_v2  # noqa: F401,E402
 from .ops.msda_fused import (  # noqa: F401,E402
     MultiScaleDeformableAttnFusedFunction,
     multi_scale_deformable_attn_fused,
 )
 
 __all__ = [
+    "GridSampler2dV2Function",
+    "grid_sampler2d_v2",
     "GeometricKernelAttentionFunc",
     "geometric_kernel_attention",
     "AdsDeformableAggregation",

@@ -28,6 +28,9 @@ EXPORTS = (
     "mxd_gka_forward",
     "mxd_gka_backward_workspace_bytes",
     "mxd_gka_backward",
+    "mxd_grid_sampler2d_forward",
+    "mxd_grid_sampler2d_backward_workspace_bytes",
+    "mxd_grid_sampler2d_backward",
 )
 
 
@@ -87,6 +90,12 @@ def load():
     lib.mxd_gka_backward_workspace_bytes.argtypes = [ci] + [i64] * 7
     lib.mxd_gka_backward.restype = ci
     lib.mxd_gka_backward.argtypes = [p] * 9 + [ctypes.c_size_t, ci] + [i64] * 7 + [p]
+    lib.mxd_grid_sampler2d_forward.restype = ci
+    lib.mxd_grid_sampler2d_forward.argtypes = [p] * 3 + [ci] + [i64] * 6 + [ci] * 3 + [p]
+    lib.mxd_grid_sampler2d_backward_workspace_bytes.restype = ctypes.c_size_t
+    lib.mxd_grid_sampler2d_backward_workspace_bytes.argtypes = [ci] + [i64] * 6
+    lib.mxd_grid_sampler2d_backward.restype = ci
+    lib.mxd_grid_sampler2d_backward.argtypes = [p] * 6 + [ctypes.c_size_t, ci] + [i64] * 6 + [ci] * 3 + [p]
     _lib = lib
     return lib
 

@@ -43,12 +43,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     if (!decode_block(a.plan, blockIdx.x, a.bs, a.nh, a.nq, &wk)) return;
 
     for (int i = threadIdx.x; i < a.nl; i += blockDim.x) {
-        i32x4 L;
-        L.x = a.shapes[2 * i];
-        L.y = a.shapes[2 * i + 1];
-        L.z = a.lsi[i];
-        L.w = 0;
-        lvl[i] = L;
+        lvl[i] = load_level(a, i);
     }
     __syncthreads();
 
@@ -86,7 +81,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             const int l = sr.l;
             const float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
             const bool inside = SRC != kSrcDagg || (cx > 0.0f && cx < 1.0f && cy > 0.0f && cy < 1.0f);
-            const Sample sm = source_geometry<SRC>(cx, cy, lvl[l], a.nk, inside);
+            const Sample sm = source_geometry<SRC>(cx, cy, lvl[l], a.nk, inside, a.grid);
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
                 if ((sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0) {
@@ -186,11 +181,12 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
                     x = to_f32(loc[2 * sr.loc_e]);
                     y = to_f32(loc[2 * sr.loc_e + 1]);
-                    aw = to_f32(attn[sr.w_e]);
+                    if constexpr (SRC == kSrcGrid) aw = 1.0f;  // no weights tensor
+                    else aw = to_f32(attn[sr.w_e]);
                     l = sr.l;
                 }
                 const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside);
+                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside, a.grid);
                 Entry en;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -278,10 +274,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
                     const float x = to_f32(loc[2 * sr.loc_e]);
                     const float y = to_f32(loc[2 * sr.loc_e + 1]);
-                    const float aw = to_f32(attn[sr.w_e]);
+                    float aw = 1.0f;
+                    if constexpr (SRC != kSrcGrid) aw = to_f32(attn[sr.w_e]);
                     const int l = sr.l;
                     const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                    const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, inside);
+                    const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, inside, a.grid);
                     const f32x4 dd = dots[u * kChunk + sl];
                     float ga = 0.f, gx = 0.f, gy = 0.f;
                     if (sm.valid) {
@@ -290,7 +287,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         gx = sm.Wf * aw * (hh * (dd[1] - dd[0]) + sm.lh * (dd[3] - dd[2]));
                         gy = sm.Hf * aw * (hw * (dd[2] - dd[0]) + sm.lw * (dd[3] - dd[1]));
                     }
-                    gattn[sr.w_e] = from_f32<T>(ga);
+                    if constexpr (SRC != kSrcGrid) gattn[sr.w_e] = from_f32<T>(ga);
                     if constexpr (SRC == kSrcDagg) {
                         // one location serves the scales of its camera and every head: sum over the
                         // scales here (neighbouring lanes), per head into a float32 partial image that a
@@ -435,7 +432,12 @@ template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
 {
     const dim3 grid(a.plan.grid), block(a.plan.block);
-    if (a.gka) {
+    if (a.grid) {
+        if (scatter)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcGrid>), grid, block, a.plan.lds_bytes, stream, a);
+        else
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcGrid>), grid, block, a.plan.lds_bytes, stream, a);
+    } else if (a.gka) {
         if (scatter)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcGka>), grid, block, a.plan.lds_bytes, stream, a);
         else

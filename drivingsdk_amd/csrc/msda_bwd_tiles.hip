@@ -55,7 +55,8 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
     int32_t total = 0;
     for (int l = 0; l < a.nl; ++l) {
         int32_t P;
-        const int32_t nt = level_tile_count(a.shapes[2 * l], a.shapes[2 * l + 1], a.lsi[l], a.nk, &P);
+        const i32x4 L = load_level(a, l);
+        const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, &P);
         const bool fits = total + nt <= a.tbl_stride - 1;
         lv_first[l] = total;
         lv_nt[l] = fits ? nt : 0;
@@ -68,7 +69,8 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
     for (int l = a.nl - 1; l >= 0; --l) {
         const int32_t nt = lv_nt[l];
         if (nt == 0) continue;
-        const int32_t H = a.shapes[2 * l], W = a.shapes[2 * l + 1], base = a.lsi[l];
+        const i32x4 L = load_level(a, l);
+        const int32_t H = L.x, W = L.y, base = L.z;
         int32_t P;
         level_tile_count(H, W, base, a.nk, &P);
         // two pair records per sample, spread evenly over the tiles of the level

@@ -334,21 +334,24 @@ int mxd_msda_decode_block(const mxd_msda_plan* plan, uint32_t block_index, int64
     return 1;
 }
 
-static int forward_common(int gka, const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+// kind: 0 multi-scale deformable attention, 1 geometric kernel attention, >= 2: grid sampler with mode kind - 1
+static int forward_common(int kind, const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
                           const void* sampling_loc, const void* attn_weight, void* output, int dtype, int64_t bs,
                           int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
-                          void* hip_stream)
+                          void* hip_stream, int64_t grid_h = 0, int64_t grid_w = 0)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
+    const int gka = kind == 1, grid = kind >= 2 ? kind - 1 : 0;
+    const char* who = grid ? "mxd_grid_sampler2d_forward" : gka ? "mxd_gka_forward" : "mxd_msda_forward";
     int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
-    if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !output)
-        return fail(MXD_E_NULL, "%s: NULL data pointer", gka ? "mxd_gka_forward" : "mxd_msda_forward");
+    if (!value || !sampling_loc || !output || (!grid && (!spatial_shapes || !level_start_index || !attn_weight)))
+        return fail(MXD_E_NULL, "%s: NULL data pointer", who);
     int align = ptr_align(value);
     if (ptr_align(output) < align) align = ptr_align(output);
     mxd::KArgs a;
     memset(&a, 0, sizeof(a));
-    int cache = gka == 0;
+    int cache = kind == 0;
     rc = make_plan(0, dtype, d, align, &a.plan, &cache);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
@@ -359,9 +362,12 @@ static int forward_common(int gka, const void* value, const int32_t* spatial_sha
     a.attn = attn_weight;
     a.out = output;
     a.gka = gka;
+    a.grid = grid;
+    a.grid_h = (int32_t)grid_h;
+    a.grid_w = (int32_t)grid_w;
     a.lds_cache_bytes = cache;
     const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
-    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", gka ? "mxd_gka_forward" : "mxd_msda_forward", hipGetErrorString(e));
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(e));
     return MXD_OK;
 }
 
@@ -379,6 +385,26 @@ int mxd_gka_forward(const void* value, const int32_t* spatial_shapes, const int3
 {
     return forward_common(1, value, spatial_shapes, level_start_index, sampling_locations, attn_weights, output, dtype,
                           bs, nk, nh, hd, nl, nl, nq, np, hip_stream);
+}
+
+static int grid_mode(int interpolation_mode, int padding_mode, int align_corners)
+{
+    if (interpolation_mode != 0) return fail(MXD_E_SHAPE, "grid_sampler2d: only bilinear interpolation (0) is built, got %d", interpolation_mode);
+    if (padding_mode != 0 && padding_mode != 1)
+        return fail(MXD_E_SHAPE, "grid_sampler2d: padding_mode must be 0 (zeros) or 1 (border), got %d", padding_mode);
+    return 1 + padding_mode + (align_corners ? 2 : 0);
+}
+
+int mxd_grid_sampler2d_forward(const void* input_nhwc, const void* grid, void* output_nhwc, int dtype, int64_t n,
+                               int64_t c, int64_t h_in, int64_t w_in, int64_t h_out, int64_t w_out,
+                               int interpolation_mode, int padding_mode, int align_corners, void* hip_stream)
+{
+    const int mode = grid_mode(interpolation_mode, padding_mode, align_corners);
+    if (mode < 0) return mode;
+    if (h_in <= 0 || w_in <= 0 || h_in * w_in >= (int64_t(1) << 31))
+        return fail(MXD_E_SHAPE, "grid_sampler2d: input of %lld x %lld pixels is beyond what this build indexes", (long long)h_in, (long long)w_in);
+    return forward_common(1 + mode, input_nhwc, nullptr, nullptr, grid, nullptr, output_nhwc, dtype, n, h_in * w_in, 1, c, 1,
+                          1, h_out * w_out, 1, hip_stream, h_in, w_in);
 }
 
 int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
@@ -421,18 +447,19 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
     return bwd_layout(dtype, d).total;
 }
 
-static int backward_common(int gka, const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+static int backward_common(int kind, const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
                            const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
                            void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype,
                            int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq,
-                           int64_t np, int flags, void* hip_stream)
+                           int64_t np, int flags, void* hip_stream, int64_t grid_h = 0, int64_t grid_w = 0)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
-    const char* who = gka ? "mxd_gka_backward" : "mxd_msda_backward";
+    const int gka = kind == 1, grid = kind >= 2 ? kind - 1 : 0;
+    const char* who = grid ? "mxd_grid_sampler2d_backward" : gka ? "mxd_gka_backward" : "mxd_msda_backward";
     int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
-    if (!value || !spatial_shapes || !level_start_index || !sampling_loc || !attn_weight || !grad_output || !grad_value ||
-        (!grad_loc && !gka) || !grad_attn)
+    if (!value || !sampling_loc || !grad_output || !grad_value || (!grad_loc && !gka) || (!grad_attn && !grid) ||
+        (!grid && (!spatial_shapes || !level_start_index || !attn_weight)))
         return fail(MXD_E_NULL, "%s: NULL data pointer", who);
     const BwdLayout L = bwd_layout(dtype, d);
     const size_t need = L.total;
@@ -469,6 +496,9 @@ static int backward_common(int gka, const void* value, const int32_t* spatial_sh
     a.grad_loc = grad_loc;
     a.grad_attn = grad_attn;
     a.gka = gka;
+    a.grid = grid;
+    a.grid_h = (int32_t)grid_h;
+    a.grid_w = (int32_t)grid_w;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * nk * nh * hd;
     hipError_t e = hipSuccess;
@@ -518,6 +548,28 @@ int mxd_gka_backward(const void* value, const int32_t* spatial_shapes, const int
     return backward_common(1, value, spatial_shapes, level_start_index, sampling_locations, attn_weights, grad_output,
                            grad_value, nullptr, grad_attn_weights, workspace, workspace_bytes, dtype, bs, nk, nh, hd, nl,
                            nl, nq, np, 0, hip_stream);
+}
+
+size_t mxd_grid_sampler2d_backward_workspace_bytes(int dtype, int64_t n, int64_t c, int64_t h_in, int64_t w_in,
+                                                   int64_t h_out, int64_t w_out)
+{
+    if (h_in <= 0 || w_in <= 0 || h_in * w_in >= (int64_t(1) << 31)) return 0;
+    return mxd_msda_backward_workspace_bytes(dtype, n, h_in * w_in, 1, c, 1, 1, h_out * w_out, 1);
+}
+
+int mxd_grid_sampler2d_backward(const void* grad_output_nhwc, const void* input_nhwc, const void* grid,
+                                void* grad_input_nhwc, void* grad_grid, void* workspace, size_t workspace_bytes,
+                                int dtype, int64_t n, int64_t c, int64_t h_in, int64_t w_in, int64_t h_out,
+                                int64_t w_out, int interpolation_mode, int padding_mode, int align_corners,
+                                void* hip_stream)
+{
+    const int mode = grid_mode(interpolation_mode, padding_mode, align_corners);
+    if (mode < 0) return mode;
+    if (h_in <= 0 || w_in <= 0 || h_in * w_in >= (int64_t(1) << 31))
+        return fail(MXD_E_SHAPE, "grid_sampler2d: input of %lld x %lld pixels is beyond what this build indexes", (long long)h_in, (long long)w_in);
+    return backward_common(1 + mode, input_nhwc, nullptr, nullptr, grid, nullptr, grad_output_nhwc, grad_input_nhwc,
+                           grad_grid, nullptr, workspace, workspace_bytes, dtype, n, h_in * w_in, 1, c, 1, 1,
+                           h_out * w_out, 1, 0, hip_stream, h_in, w_in);
 }
 
 int mxd_dagg_forward(const void* mc_ms_feat, const int32_t* spatial_shape, const int32_t* scale_start_index,

@@ -35,6 +35,8 @@ struct KArgs {
     int32_t scales;
     uint32_t sc_magic;     // ceil(2^20/scales): level / scales
     int32_t lds_cache_bytes;  // forward: LDS set aside for the rows of the last (coarsest) levels, 0 = none
+    int32_t grid_h, grid_w;  // grid sampler: the one level's shape comes with the call, not from device memory
+    int32_t grid;          // grid sampler: 1 + padding mode (0 zeros, 1 border) + 2*align_corners; 0 = not a grid sampler
     int32_t gka;           // geometric kernel attention: locations are pixel indices, one pixel per sample
     int32_t sc_pow2;       // scales is a power of two that divides 16: location gradients are summed over the
                            // scales across lanes and stored once; otherwise they are added with atomics
@@ -62,8 +64,15 @@ struct KArgs {
     mxd_msda_plan plan;
 };
 
+// Level l as {H, W, level_start_index, 0}.
+__device__ inline i32x4 load_level(const KArgs& a, int l)
+{
+    if (a.grid) return i32x4{a.grid_h, a.grid_w, 0, 0};
+    return i32x4{a.shapes[2 * l], a.shapes[2 * l + 1], a.lsi[l], 0};
+}
+
 // Where a kernel takes the location and the weight of sample s of unit (b, q, h) from.
-enum : int { kSrcPlain = 0, kSrcFused = 1, kSrcDagg = 2, kSrcGka = 3 };
+enum : int { kSrcPlain = 0, kSrcFused = 1, kSrcDagg = 2, kSrcGka = 3, kSrcGrid = 4 };
 struct SampleRef {
     int64_t loc_e;  // index of the (x, y) pair
     int64_t w_e;    // index of the weight
@@ -305,9 +314,59 @@ __device__ inline Sample gka_geometry(float x, float y, i32x4 level, int32_t nk,
     return s;
 }
 
-template <int SRC>
-__device__ inline Sample source_geometry(float x, float y, i32x4 level, int32_t nk, bool active)
+// 2-D grid sampler, bilinear (reference: mx_driving/ops/grid_sampler2d_v2.py; the arithmetic is that of
+// torch.nn.functional.grid_sample, which the reference's test uses as its golden): the location is a grid coordinate in
+// [-1, 1], mapped to pixels by ((g+1)/2)*(size-1) with align_corners and ((g+1)*size-1)/2 without, clipped to
+// [0, size-1] for border padding (the gradient is zero where it clips); Wf / Hf carry d(pixel)/d(grid).
+__device__ inline Sample grid_geometry(float gx, float gy, i32x4 level, int32_t nk, bool active, int mode)
 {
+#pragma clang fp contract(off)
+    Sample s;
+    const int32_t H = level.x, W = level.y, base = level.z;
+    const bool border = (mode - 1) & 1, align = (mode - 1) & 2;
+    float ix, iy;
+    if (align) {
+        ix = ((gx + 1.0f) / 2.0f) * (float)(W - 1);
+        iy = ((gy + 1.0f) / 2.0f) * (float)(H - 1);
+        s.Wf = (float)(W - 1) / 2.0f;
+        s.Hf = (float)(H - 1) / 2.0f;
+    } else {
+        ix = ((gx + 1.0f) * (float)W - 1.0f) / 2.0f;
+        iy = ((gy + 1.0f) * (float)H - 1.0f) / 2.0f;
+        s.Wf = (float)W / 2.0f;
+        s.Hf = (float)H / 2.0f;
+    }
+    if (border) {
+        if (ix <= 0.0f) { ix = 0.0f; s.Wf = 0.0f; } else if (ix >= (float)(W - 1)) { ix = (float)(W - 1); s.Wf = 0.0f; }
+        if (iy <= 0.0f) { iy = 0.0f; s.Hf = 0.0f; } else if (iy >= (float)(H - 1)) { iy = (float)(H - 1); s.Hf = 0.0f; }
+    }
+    s.valid = active && (ix > -1.0f) && (iy > -1.0f) && (ix < (float)W) && (iy < (float)H);  // false for NaN
+    const float fx = __builtin_floorf(ix), fy = __builtin_floorf(iy);
+    s.lw = ix - fx;
+    s.lh = iy - fy;
+    const int32_t x0 = s.valid ? (int32_t)fx : 0, y0 = s.valid ? (int32_t)fy : 0;
+    const float hw = 1.0f - s.lw, hh = 1.0f - s.lh;
+    const bool vx0 = (uint32_t)x0 < (uint32_t)W, vx1 = (uint32_t)(x0 + 1) < (uint32_t)W;
+    const bool vy0 = (uint32_t)y0 < (uint32_t)H, vy1 = (uint32_t)(y0 + 1) < (uint32_t)H;
+    const int32_t p00 = base + y0 * W + x0;
+    s.pix[0] = p00;
+    s.pix[1] = p00 + 1;
+    s.pix[2] = p00 + W;
+    s.pix[3] = p00 + W + 1;
+    const bool cv[4] = {vy0 && vx0, vy0 && vx1, vy1 && vx0, vy1 && vx1};
+    const float wt[4] = {hh * hw, hh * s.lw, s.lh * hw, s.lh * s.lw};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        s.cvalid[k] = s.valid && cv[k] && ((uint32_t)s.pix[k] < (uint32_t)nk);
+        s.w[k] = s.valid ? wt[k] : 0.0f;
+    }
+    return s;
+}
+
+template <int SRC>
+__device__ inline Sample source_geometry(float x, float y, i32x4 level, int32_t nk, bool active, int grid_mode = 0)
+{
+    if constexpr (SRC == kSrcGrid) return grid_geometry(x, y, level, nk, active, grid_mode);
     if constexpr (SRC == kSrcGka) return gka_geometry(x, y, level, nk, active);
     else return sample_geometry(x, y, level, nk, active);
 }

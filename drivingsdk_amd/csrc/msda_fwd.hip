@@ -31,6 +31,8 @@
 // kernels/deformable_aggregation/): the same sum with a channel group as head, a (camera, scale) pair as
 // level, one location per (anchor, point, camera) shared by scales and groups, weights laid out
 // [.., point, camera, scale, group], and samples counted only strictly inside (0, 1) x (0, 1).
+// SRC = kSrcGka: geometric kernel attention (the location is a clamped pixel index, one row per sample).
+// SRC = kSrcGrid: bilinear 2-D grid sampler (one level, one head, one point, weight 1, grid coordinates).
 #include "msda_device.h"
 
 namespace mxd {
@@ -48,12 +50,7 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
     if (!decode_block(a.plan, blockIdx.x, a.bs, a.nh, a.nq, &wk)) return;      // whole workgroup leaves
 
     for (int i = threadIdx.x; i < a.nl; i += blockDim.x) {
-        i32x4 L;
-        L.x = a.shapes[2 * i];
-        L.y = a.shapes[2 * i + 1];
-        L.z = a.lsi[i];
-        L.w = 0;
-        lvl[i] = L;
+        lvl[i] = load_level(a, i);
     }
     __syncthreads();
 
@@ -174,7 +171,8 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
                     const SampleRef r = sample_ref<SRC>(a, wk.b, q, wk.h, s);
                     x = to_f32(loc[2 * r.loc_e]);
                     y = to_f32(loc[2 * r.loc_e + 1]);
-                    aw = to_f32(attn[r.w_e]);
+                    if constexpr (SRC == kSrcGrid) aw = 1.0f;  // no weights tensor
+                    else aw = to_f32(attn[r.w_e]);
                     l = r.l;
                     if constexpr (FUSED) {
                         const T* rp = ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim;
@@ -190,7 +188,7 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
                 }
                 // deformable aggregation samples only strictly inside the image (0 < x, y < 1)
                 const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside);
+                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside, a.grid);
                 Entry en;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
@@ -273,7 +271,9 @@ template <typename T, int VEC, int NPASS>
 static hipError_t launch_one(const KArgs& a, hipStream_t stream)
 {
     const dim3 grid(a.plan.grid), block(a.plan.block);
-    if (a.gka)
+    if (a.grid)
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcGrid, false>), grid, block, a.plan.lds_bytes, stream, a);
+    else if (a.gka)
         hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcGka, false>), grid, block, a.plan.lds_bytes, stream, a);
     else if (a.cams > 0)
         hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcDagg, false>), grid, block, a.plan.lds_bytes, stream, a);

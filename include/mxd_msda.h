@@ -206,6 +206,25 @@ int mxd_gka_backward(const void* value, const int32_t* spatial_shapes, const int
                      int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nq, int64_t np,
                      void* hip_stream);
 
+/* ---- 2-D grid sampler, bilinear ----------------------------------------------------------------
+ * Replaces the aclnnGridSampler2dV2 / aclnnGridSampler2dV2Grad launches of grid_sampler2d_v2 and
+ * grid_sampler2d_v2_backward (mx_driving/csrc/GridSampler2dV2.cpp:33-99), which, like these entry points, work
+ * on channel-last tensors (the binding permutes NCHW <-> NHWC around them, :68-76):
+ *   input_nhwc [n, h_in, w_in, c]   grid [n, h_out, w_out, 2] = (x, y) in [-1, 1]   output_nhwc [n, h_out, w_out, c]
+ * with the arithmetic of torch.nn.functional.grid_sample (the reference's golden): interpolation_mode 0 (bilinear),
+ * padding_mode 0 (zeros) or 1 (border), align_corners 0/1.  c <= 256. */
+int mxd_grid_sampler2d_forward(const void* input_nhwc, const void* grid, void* output_nhwc, int dtype, int64_t n,
+                               int64_t c, int64_t h_in, int64_t w_in, int64_t h_out, int64_t w_out,
+                               int interpolation_mode, int padding_mode, int align_corners, void* hip_stream);
+size_t mxd_grid_sampler2d_backward_workspace_bytes(int dtype, int64_t n, int64_t c, int64_t h_in, int64_t w_in,
+                                                   int64_t h_out, int64_t w_out);
+/* grad_input_nhwc [n, h_in, w_in, c] and grad_grid [n, h_out, w_out, 2]; every element is written. */
+int mxd_grid_sampler2d_backward(const void* grad_output_nhwc, const void* input_nhwc, const void* grid,
+                                void* grad_input_nhwc, void* grad_grid, void* workspace, size_t workspace_bytes,
+                                int dtype, int64_t n, int64_t c, int64_t h_in, int64_t w_in, int64_t h_out,
+                                int64_t w_out, int interpolation_mode, int padding_mode, int align_corners,
+                                void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,8 +12,10 @@ from drivingsdk_amd.ops.deformable_aggregation import (  # noqa: F401,E402  (mx_
     npu_deformable_aggregation,
 )
 from drivingsdk_amd.ops.geometric_kernel_attention import geometric_kernel_attention  # noqa: F401,E402
+from drivingsdk_amd.ops.grid_sampler2d_v2 import grid_sampler2d_v2  # noqa: F401,E402
 
 __all__ = [
+    "grid_sampler2d_v2",
     "geometric_kernel_attention",
     "deformable_aggregation",
     "npu_deformable_aggregation",

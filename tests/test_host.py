@@ -16,7 +16,7 @@ from drivingsdk_amd import _C, _lib, workloads
 def test_library_exports_every_declared_symbol():
     with open(os.path.join(ROOT, "include", "mxd_msda.h")) as f:
         header = f.read()
-    declared = set(re.findall(r"\b(mxd_(?:msda|dagg|gka)_[a-z_]+)\s*\(", header))
+    declared = set(re.findall(r"\b(mxd_(?:msda|dagg|gka|grid_sampler2d)_[a-z_]+)\s*\(", header))
     declared.discard("mxd_msda_plan")
     assert declared == set(_lib.EXPORTS)
     lib = _lib.load()
