@@ -81,7 +81,8 @@ def _kernel_times(d, iters, warmup):
 def _module_forward_times(d, iters, warmup):
     """The step either side of the operator in the calling module (softmax of the logits, location =
     reference point + offset / (W, H)): torch element-wise kernels followed by the operator, against the
-    fused forward in which both happen inside the kernel.  Same synthetic module inputs for both."""
+    fused form in which both -- and their chain rule in the backward -- happen inside the kernels.  Same
+    synthetic module inputs for both; forward alone, then forward + backward through autograd."""
     import torch
 
     import drivingsdk_amd
@@ -104,7 +105,28 @@ def _module_forward_times(d, iters, warmup):
                                                                 off, logits)
 
     with torch.no_grad():
-        return {"unfused_ms": _event_ms(unfused, iters, warmup), "fused_ms": _event_ms(fused, iters, warmup)}
+        res = {"unfused_ms": _event_ms(unfused, iters, warmup), "fused_ms": _event_ms(fused, iters, warmup)}
+
+    # forward + backward of the same two forms, gradients for value, reference points, offsets and logits
+    leaves = [t.detach().clone().requires_grad_() for t in (d.value, ref, off, logits)]
+    grad_out = torch.randn(bs, nq, nh * hd, generator=g).to(dev)
+
+    def train(form):
+        def run():
+            v, r, o, z = leaves
+            for t in leaves:
+                t.grad = None
+            if form == "unfused":
+                loc, attn = msda_fused.sampling_inputs(d.spatial_shapes, r, o, z)
+                out = drivingsdk_amd.multi_scale_deformable_attn(v, d.spatial_shapes, d.level_start_index, loc, attn)
+            else:
+                out = drivingsdk_amd.multi_scale_deformable_attn_fused(v, d.spatial_shapes, d.level_start_index, r, o, z)
+            out.backward(grad_out)
+        return run
+
+    res["unfused_fwd_bwd_ms"] = _event_ms(train("unfused"), iters, warmup)
+    res["fused_fwd_bwd_ms"] = _event_ms(train("fused"), iters, warmup)
+    return res
 
 
 def _committed_traffic(workload, dtype):

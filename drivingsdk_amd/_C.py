@@ -162,6 +162,65 @@ def msda_fused_forward(value, value_spatial_shapes, value_level_start_index, ref
     return output
 
 
+def msda_fused_backward(value, value_spatial_shapes, value_level_start_index, reference_points, sampling_offsets,
+                        attention_logits, output, grad_output, need_grad_reference_points=True):
+    """Backward of ``msda_fused_forward`` (``mxd_msda_fused_backward``): the chain rule through the softmax and the
+    sampling-location arithmetic runs inside the operator's first backward kernel.  ``output`` is the forward
+    result.  Returns ``(grad_value, grad_reference_points or None, grad_sampling_offsets, grad_attention_logits)``,
+    each with the shape and dtype of its input."""
+    _check(value.dtype in _FLOAT_CODES,
+           f"value: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {value.dtype}")
+    _check(value.dim() == 4 and sampling_offsets.dim() == 6 and sampling_offsets.size(5) == 2,
+           "msda_fused_backward: expected value [bs, nk, nh, hd] and sampling_offsets [bs, nq, nh, nl, np, 2]")
+    bs, nk, nh, hd = value.shape
+    _, nq, _, nl, npts, _ = sampling_offsets.shape
+    _check(tuple(value_spatial_shapes.shape) == (nl, 2) and value_level_start_index.numel() == nl,
+           "value_spatial_shapes / value_level_start_index: expected the levels of sampling_offsets")
+    _check(value_spatial_shapes.dtype == torch.int32 and value_level_start_index.dtype == torch.int32,
+           "value_spatial_shapes / value_level_start_index: int32 tensors expected")
+    _check(sampling_offsets.size(0) == bs and sampling_offsets.size(2) == nh,
+           "sampling_offsets: batch size / num_heads do not match value")
+    _check(reference_points.dim() == 4 and tuple(reference_points.shape[:3]) == (bs, nq, nl),
+           "reference_points: expected [bs, num_queries, num_levels, 2 or 4]")
+    ref_dim = reference_points.size(3)
+    _check(ref_dim in (2, 4), f"Last dim of reference_points must be 2 or 4, but get {ref_dim} instead.")
+    _check(attention_logits.numel() == bs * nq * nh * nl * npts and attention_logits.size(0) == bs,
+           "attention_logits: expected [bs, num_queries, num_heads, num_levels*num_points]")
+    _check(output.numel() == bs * nq * nh * hd and grad_output.numel() == bs * nq * nh * hd,
+           "output / grad_output: expected [bs, num_queries, num_heads*embed_dims]")
+    tensors = (value, value_spatial_shapes, value_level_start_index, reference_points, sampling_offsets,
+               attention_logits, output, grad_output)
+    _check(all(t.is_cuda for t in tensors),
+           "msda_fused_backward: all tensors must live on a GPU (this build has no CPU implementation)")
+    _check(all(t.device == value.device for t in tensors), "msda_fused_backward: tensors are on different devices")
+    lib = _lib.load()
+    dt = value.dtype
+    code = _FLOAT_CODES[dt]
+    value = value.contiguous()
+    shapes, lsi = value_spatial_shapes.contiguous(), value_level_start_index.contiguous()
+    ref = reference_points.to(dt).contiguous()
+    off = sampling_offsets.to(dt).contiguous()
+    logits = attention_logits.to(dt).contiguous()
+    out = output.to(dt).contiguous()
+    gout = grad_output.to(dt).contiguous()
+    grad_value = torch.empty_like(value)
+    grad_off = torch.empty_like(off)
+    grad_logits = torch.empty_like(logits)
+    grad_ref = torch.empty_like(ref) if need_grad_reference_points else None
+    want = 1 if need_grad_reference_points else 0
+    ws_bytes = lib.mxd_msda_fused_backward_workspace_bytes(code, bs, nk, nh, hd, nl, nq, npts, ref_dim, want)
+    workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=value.device)
+    with torch.cuda.device(value.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib.mxd_msda_fused_backward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), ref.data_ptr(), ref_dim,
+                                         off.data_ptr(), logits.data_ptr(), out.data_ptr(), gout.data_ptr(),
+                                         grad_value.data_ptr(), grad_ref.data_ptr() if want else None,
+                                         grad_off.data_ptr(), grad_logits.data_ptr(), workspace.data_ptr(), ws_bytes,
+                                         code, bs, nk, nh, hd, nl, nq, npts, 0, stream)
+    _check(rc == 0, _lib.last_error() if rc != 0 else "")
+    return grad_value, grad_ref, grad_off, grad_logits
+
+
 # ---- deformable aggregation (mx_driving/csrc/DeformableAggregation.cpp:20-82 of the reference) --------------
 
 def _dagg_check(mc_ms_feat, spatial_shape, scale_start_index, sampling_location, weights, name):

@@ -20,6 +20,8 @@ EXPORTS = (
     "mxd_msda_decode_block",
     "mxd_msda_forward",
     "mxd_msda_fused_forward",
+    "mxd_msda_fused_backward_workspace_bytes",
+    "mxd_msda_fused_backward",
     "mxd_msda_backward_workspace_bytes",
     "mxd_msda_backward",
     "mxd_dagg_forward",
@@ -74,6 +76,10 @@ def load():
     lib.mxd_msda_forward.argtypes = [p] * 6 + [ci] + [i64] * 8 + [p]
     lib.mxd_msda_fused_forward.restype = ci
     lib.mxd_msda_fused_forward.argtypes = [p] * 4 + [ci] + [p] * 3 + [ci] + [i64] * 7 + [p]
+    lib.mxd_msda_fused_backward_workspace_bytes.restype = ctypes.c_size_t
+    lib.mxd_msda_fused_backward_workspace_bytes.argtypes = [ci] + [i64] * 7 + [ci, ci]
+    lib.mxd_msda_fused_backward.restype = ci
+    lib.mxd_msda_fused_backward.argtypes = [p] * 4 + [ci] + [p] * 9 + [ctypes.c_size_t, ci] + [i64] * 7 + [ci, p]
     lib.mxd_msda_backward_workspace_bytes.restype = ctypes.c_size_t
     lib.mxd_msda_backward_workspace_bytes.argtypes = [ci] + [i64] * 8
     lib.mxd_msda_backward.restype = ci

@@ -36,6 +36,7 @@ template <typename T, int VEC, int NPASS, bool SCATTER, int SRC>
 __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
     constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
+    constexpr bool FUSED = SRC == kSrcFused;
 
     extern __shared__ __align__(16) unsigned char smem[];
     i32x4* lvl = reinterpret_cast<i32x4*>(smem);
@@ -79,7 +80,10 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             const int qr = i / a.S, s = i - qr * a.S;
             const SampleRef sr = sample_ref<SRC>(a, wk.b, wk.q_begin + qr, wk.h, s);
             const int l = sr.l;
-            const float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
+            float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
+            if constexpr (FUSED)
+                fused_location(a, static_cast<const T*>(a.ref) + (((int64_t)wk.b * a.nq + wk.q_begin + qr) * a.nl + l) * a.ref_dim,
+                               lvl[l], cx, cy);
             const bool inside = SRC != kSrcDagg || (cx > 0.0f && cx < 1.0f && cy > 0.0f && cy < 1.0f);
             const Sample sm = source_geometry<SRC>(cx, cy, lvl[l], a.nk, inside, a.grid);
 #pragma unroll
@@ -133,6 +137,10 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     const T* gout = static_cast<const T*>(a.grad_out);
     T* gloc = static_cast<T*>(a.grad_loc);
     T* gattn = static_cast<T*>(a.grad_attn);
+    const T* ref = static_cast<const T*>(a.ref);
+    // fused form: per unit {max logit, sum of exponentials, <forward row, grad_out row>} in the pad entry that
+    // ends the unit's staging strip
+    auto unit_stats = [&](int u) { return reinterpret_cast<float*>(stage + u * kChunkStride + kChunk); };
 
     const __amdgpu_buffer_rsrc_t vres =
         make_rsrc(static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes, a.batch_bytes);
@@ -169,6 +177,44 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             }
         }
 
+        if constexpr (FUSED) {
+            // softmax backward: grad_logit_s = w_s * (grad_w_s - sum_t w_t * grad_w_t), and the sum over the
+            // unit's samples equals the dot product of the forward row with the grad_out row
+            const T* orow = static_cast<const T*>(a.out) +
+                            (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
+            float dsum = 0.0f;
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p) {
+                const int ch = (c + p * LPR) * VEC;
+                if (unit_ok && ch < a.hd) {
+                    float ov[VEC];
+                    RowIO<T, VEC>::load_global(orow + ch, ov);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) dsum = __builtin_fmaf(ov[e], gv[p][e], dsum);
+                }
+            }
+            for (int d = 1; d < LPR; d <<= 1) dsum += __shfl_xor(dsum, d, kWave);
+            if (c == 0 && g < U) unit_stats(g)[2] = dsum;
+            // softmax statistics: lanes 16u..16u+15 share unit u, each takes every 16th logit
+            for (int i = lane; i < entries; i += kWave) {
+                const int u = i >> 4, sl = i & (kChunk - 1), q = q0 + u;
+                const T* lg = attn + (((int64_t)wk.b * a.nq + (q < wk.q_end ? q : wk.q_begin)) * a.nh + wk.h) * a.S_full;
+                float m = -__builtin_inff();
+                for (int s = sl; s < a.S; s += kChunk) m = __builtin_fmaxf(m, to_f32(lg[s]));
+#pragma unroll
+                for (int d = 1; d < kChunk; d <<= 1) m = __builtin_fmaxf(m, __shfl_xor(m, d, kWave));
+                float sum = 0.0f;
+                for (int s = sl; s < a.S; s += kChunk) sum += expf(to_f32(lg[s]) - m);
+#pragma unroll
+                for (int d = 1; d < kChunk; d <<= 1) sum += __shfl_xor(sum, d, kWave);
+                if (sl == 0) {
+                    unit_stats(u)[0] = m;
+                    unit_stats(u)[1] = sum;
+                }
+            }
+            wave_lds_sync();
+        }
+
         for (int c0 = 0; c0 < a.S; c0 += kChunk) {
             // ---- geometry -----------------------------------------------------------------
             for (int i = lane; i < entries; i += kWave) {
@@ -184,6 +230,10 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     if constexpr (SRC == kSrcGrid) aw = 1.0f;  // no weights tensor
                     else aw = to_f32(attn[sr.w_e]);
                     l = sr.l;
+                    if constexpr (FUSED) {
+                        fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim, lvl[l], x, y);
+                        aw = expf(aw - unit_stats(u)[0]) / unit_stats(u)[1];
+                    }
                 }
                 const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
                 const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside, a.grid);
@@ -272,11 +322,18 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 const int s = c0 + sl, q = q0 + u;
                 if ((q < wk.q_end) && (s < a.S)) {
                     const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
-                    const float x = to_f32(loc[2 * sr.loc_e]);
-                    const float y = to_f32(loc[2 * sr.loc_e + 1]);
+                    float x = to_f32(loc[2 * sr.loc_e]);
+                    float y = to_f32(loc[2 * sr.loc_e + 1]);
                     float aw = 1.0f;
                     if constexpr (SRC != kSrcGrid) aw = to_f32(attn[sr.w_e]);
                     const int l = sr.l;
+                    const float ox = x, oy = y;  // raw offsets (fused form)
+                    const T* rp = nullptr;
+                    if constexpr (FUSED) {
+                        rp = ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim;
+                        fused_location(a, rp, lvl[l], x, y);
+                        aw = expf(aw - unit_stats(u)[0]) / unit_stats(u)[1];
+                    }
                     const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
                     const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, inside, a.grid);
                     const f32x4 dd = dots[u * kChunk + sl];
@@ -287,8 +344,51 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         gx = sm.Wf * aw * (hh * (dd[1] - dd[0]) + sm.lh * (dd[3] - dd[2]));
                         gy = sm.Hf * aw * (hw * (dd[2] - dd[0]) + sm.lw * (dd[3] - dd[1]));
                     }
-                    if constexpr (SRC != kSrcGrid) gattn[sr.w_e] = from_f32<T>(ga);
-                    if constexpr (SRC == kSrcDagg) {
+                    if constexpr (FUSED) {
+                        // chain rule through the softmax and through location = reference + offset * scale
+                        gattn[sr.w_e] = from_f32<T>(aw * (ga - unit_stats(u)[2]));
+                        float r2 = 0.0f, r3 = 0.0f;  // boxes: gradient of (w, h)
+                        if (a.ref_dim == 2) {
+                            gloc[2 * sr.loc_e] = from_f32<T>(gx / (float)lvl[l].y);
+                            gloc[2 * sr.loc_e + 1] = from_f32<T>(gy / (float)lvl[l].x);
+                        } else {
+                            gloc[2 * sr.loc_e] = from_f32<T>(gx / (float)a.np * to_f32(rp[2]) * 0.5f);
+                            gloc[2 * sr.loc_e + 1] = from_f32<T>(gy / (float)a.np * to_f32(rp[3]) * 0.5f);
+                            r2 = gx * (ox / (float)a.np * 0.5f);
+                            r3 = gy * (oy / (float)a.np * 0.5f);
+                        }
+                        if (a.grad_ref != nullptr) {
+                            // the points of a level share the reference point: sum over them here, per head
+                            // into a float32 partial image that a small kernel adds up over the heads
+                            float* part = a.grad_ref + (((int64_t)wk.h * a.bs + wk.b) * a.nq + q) * (a.nl * a.ref_dim) +
+                                          l * a.ref_dim;
+                            if (a.np_pow2) {
+                                for (int d = 1; d < a.np; d <<= 1) {
+                                    gx += __shfl_xor(gx, d, kWave);
+                                    gy += __shfl_xor(gy, d, kWave);
+                                    r2 += __shfl_xor(r2, d, kWave);
+                                    r3 += __shfl_xor(r3, d, kWave);
+                                }
+                                if ((s & (a.np - 1)) == 0) {
+                                    part[0] = gx;
+                                    part[1] = gy;
+                                    if (a.ref_dim == 4) {
+                                        part[2] = r2;
+                                        part[3] = r3;
+                                    }
+                                }
+                            } else {
+                                unsafeAtomicAdd(part, gx);
+                                unsafeAtomicAdd(part + 1, gy);
+                                if (a.ref_dim == 4) {
+                                    unsafeAtomicAdd(part + 2, r2);
+                                    unsafeAtomicAdd(part + 3, r3);
+                                }
+                            }
+                        }
+                    } else if constexpr (SRC != kSrcGrid) gattn[sr.w_e] = from_f32<T>(ga);
+                    if constexpr (FUSED) {
+                    } else if constexpr (SRC == kSrcDagg) {
                         // one location serves the scales of its camera and every head: sum over the
                         // scales here (neighbouring lanes), per head into a float32 partial image that a
                         // small kernel adds up over the heads afterwards
@@ -447,6 +547,11 @@ static hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcDagg>), grid, block, a.plan.lds_bytes, stream, a);
         else
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcDagg>), grid, block, a.plan.lds_bytes, stream, a);
+    } else if (a.ref != nullptr) {
+        if (scatter)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcFused>), grid, block, a.plan.lds_bytes, stream, a);
+        else
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcFused>), grid, block, a.plan.lds_bytes, stream, a);
     } else {
         if (scatter)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcPlain>), grid, block, a.plan.lds_bytes, stream, a);

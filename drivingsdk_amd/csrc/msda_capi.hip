@@ -447,22 +447,43 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
     return bwd_layout(dtype, d).total;
 }
 
+// What the fused form adds to a backward call.
+struct FusedBackward {
+    const void* ref;
+    int ref_dim;
+    const void* out;   // forward result
+    void* grad_ref;    // may be nullptr
+};
+
+static size_t fused_part_bytes(const Dims& d, int ref_dim)
+{
+    return (((size_t)d.nh * d.bs * d.nq * d.nl * ref_dim * sizeof(float)) + 15) & ~(size_t)15;
+}
+
 static int backward_common(int kind, const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
                            const void* sampling_loc, const void* attn_weight, const void* grad_output, void* grad_value,
                            void* grad_loc, void* grad_attn, void* workspace, size_t workspace_bytes, int dtype,
                            int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq,
-                           int64_t np, int flags, void* hip_stream, int64_t grid_h = 0, int64_t grid_w = 0)
+                           int64_t np, int flags, void* hip_stream, int64_t grid_h = 0, int64_t grid_w = 0,
+                           const FusedBackward* fused = nullptr)
 {
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     const int gka = kind == 1, grid = kind >= 2 ? kind - 1 : 0;
-    const char* who = grid ? "mxd_grid_sampler2d_backward" : gka ? "mxd_gka_backward" : "mxd_msda_backward";
+    const char* who = fused  ? "mxd_msda_fused_backward"
+                      : grid ? "mxd_grid_sampler2d_backward"
+                      : gka  ? "mxd_gka_backward"
+                             : "mxd_msda_backward";
     int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
     if (!value || !sampling_loc || !grad_output || !grad_value || (!grad_loc && !gka) || (!grad_attn && !grid) ||
         (!grid && (!spatial_shapes || !level_start_index || !attn_weight)))
         return fail(MXD_E_NULL, "%s: NULL data pointer", who);
+    if (fused && (!fused->ref || !fused->out)) return fail(MXD_E_NULL, "%s: NULL data pointer", who);
+    if (fused && fused->ref_dim != 2 && fused->ref_dim != 4)
+        return fail(MXD_E_SHAPE, "Last dim of reference_points must be 2 or 4, but get %d instead.", fused->ref_dim);
     const BwdLayout L = bwd_layout(dtype, d);
-    const size_t need = L.total;
+    const size_t part_bytes = (fused && fused->grad_ref) ? fused_part_bytes(d, fused->ref_dim) : 0;
+    const size_t need = L.total + part_bytes;
     if (need > 0 && (!workspace || workspace_bytes < need))
         return fail(MXD_E_WORKSPACE, "%s: workspace of %zu bytes required, %zu given", who, need,
                     workspace ? workspace_bytes : (size_t)0);
@@ -499,10 +520,20 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     a.grid = grid;
     a.grid_h = (int32_t)grid_h;
     a.grid_w = (int32_t)grid_w;
+    float* part = nullptr;
+    if (fused) {
+        a.ref = fused->ref;
+        a.ref_dim = fused->ref_dim;
+        a.out = const_cast<void*>(fused->out);
+        a.np_pow2 = (np & (np - 1)) == 0 && np <= 16;
+        if (part_bytes > 0) part = reinterpret_cast<float*>(ws + L.total);
+        a.grad_ref = part;
+    }
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * nk * nh * hd;
     hipError_t e = hipSuccess;
     if (!(flags & MXD_BWD_ACCUMULATE)) e = mxd::launch_fill_zero(image, n, stream);
+    if (e == hipSuccess && part && !a.np_pow2) e = mxd::launch_fill_zero(part, part_bytes / sizeof(float), stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: zero-fill launch failed: %s", who, hipGetErrorString(e));
     const bool atomic_mode = !L.tiles;
     e = mxd::launch_backward(dtype, a, atomic_mode, stream);
@@ -519,7 +550,32 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
         e = mxd::launch_round(dtype, image, grad_value, n, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: rounding launch failed: %s", who, hipGetErrorString(e));
     }
+    if (part) {
+        e = mxd::launch_sum_heads(dtype, part, fused->grad_ref, (size_t)bs * nq * nl * fused->ref_dim, (int)nh, stream);
+        if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: head sum launch failed: %s", who, hipGetErrorString(e));
+    }
     return MXD_OK;
+}
+
+size_t mxd_msda_fused_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd,
+                                               int64_t nl, int64_t nq, int64_t np, int ref_dim, int want_grad_ref)
+{
+    const Dims d{bs, nk, nh, hd, nl, nl, nq, np};
+    if (check_dims(dtype, d) != MXD_OK || (ref_dim != 2 && ref_dim != 4)) return 0;
+    return bwd_layout(dtype, d).total + (want_grad_ref ? fused_part_bytes(d, ref_dim) : 0);
+}
+
+int mxd_msda_fused_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                            const void* reference_points, int ref_dim, const void* sampling_offsets,
+                            const void* attn_logits, const void* output, const void* grad_output, void* grad_value,
+                            void* grad_reference_points, void* grad_sampling_offsets, void* grad_attn_logits,
+                            void* workspace, size_t workspace_bytes, int dtype, int64_t bs, int64_t nk, int64_t nh,
+                            int64_t hd, int64_t nl, int64_t nq, int64_t np, int flags, void* hip_stream)
+{
+    const FusedBackward f{reference_points, ref_dim, output, grad_reference_points};
+    return backward_common(0, value, spatial_shapes, level_start_index, sampling_offsets, attn_logits, grad_output,
+                           grad_value, grad_sampling_offsets, grad_attn_logits, workspace, workspace_bytes, dtype, bs,
+                           nk, nh, hd, nl, nl, nq, np, flags, hip_stream, 0, 0, &f);
 }
 
 int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,

@@ -44,6 +44,12 @@ struct KArgs {
     float* grad_value;     // fp32 accumulation image of grad_value
     void* grad_loc;
     void* grad_attn;
+    // fused form, backward: `out` holds the forward result (the softmax backward needs, per (query, head), the
+    // dot product of its row with the grad_out row); grad_loc / grad_attn receive the gradients of the offsets
+    // and of the logits; the reference points' gradient is summed over points here and over heads afterwards
+    float* grad_ref;       // [nh][bs, nq, nl, ref_dim] float32 per-head partial sums, or nullptr: not wanted
+    int32_t np_pow2;       // np is a power of two that divides 16: the point sum is taken across lanes and
+                           // stored once; otherwise added with atomics into the zero-filled partial sums
     // Hand-over from the first backward kernel to the grad_value pass.  Every workgroup of the
     // first kernel (tile_q queries of one (batch, head)) owns a slab of rec_cap pair records,
     // which it fills sorted by tile; row [w] of the table holds the start of every tile's run
@@ -146,6 +152,21 @@ template <typename T>
 __device__ inline T from_f32(float v)
 {
     return (T)v;
+}
+
+// Fused form: sampling location from the raw offset (x, y) of a sample on level `lv` = {H, W, ..}.
+// rp: the query's reference point on that level, (cx, cy) or a box (cx, cy, w, h).
+//   points: location = reference + offset / (W, H)          boxes: location = centre + offset / np * (w, h) / 2
+template <typename T>
+__device__ inline void fused_location(const KArgs& a, const T* rp, const i32x4 lv, float& x, float& y)
+{
+    if (a.ref_dim == 2) {
+        x = to_f32(rp[0]) + x / (float)lv.y;
+        y = to_f32(rp[1]) + y / (float)lv.x;
+    } else {
+        x = to_f32(rp[0]) + x / (float)a.np * to_f32(rp[2]) * 0.5f;
+        y = to_f32(rp[1]) + y / (float)a.np * to_f32(rp[3]) * 0.5f;
+    }
 }
 
 // ---- row access: VEC elements of T at a byte offset of a bound buffer -> fp32 -------------

@@ -175,14 +175,7 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
                     else aw = to_f32(attn[r.w_e]);
                     l = r.l;
                     if constexpr (FUSED) {
-                        const T* rp = ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim;
-                        if (a.ref_dim == 2) {
-                            x = to_f32(rp[0]) + x / (float)lvl[l].y;
-                            y = to_f32(rp[1]) + y / (float)lvl[l].x;
-                        } else {
-                            x = to_f32(rp[0]) + x / (float)a.np * to_f32(rp[2]) * 0.5f;
-                            y = to_f32(rp[1]) + y / (float)a.np * to_f32(rp[3]) * 0.5f;
-                        }
+                        fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim, lvl[l], x, y);
                         aw = expf(aw - stats[2 * u]) / stats[2 * u + 1];
                     }
                 }

@@ -11,9 +11,9 @@ model_examples/BEVFormer/bev_former_config.patch:404-421) run, between their lin
     output = multi_scale_deformable_attn(value, shapes, level_start_index, sampling_locations, attention_weights)
 
 ``multi_scale_deformable_attn_fused`` takes the module's raw tensors instead.  Its forward is ONE kernel in which
-locations and weights never reach memory.  Its backward evaluates the three lines above with torch (they are
-cheap element-wise work), runs the operator's own backward kernels on the result and lets autograd carry the
-gradients through the three lines -- gradients for value, reference points, offsets and logits.
+locations and weights never reach memory.  Its backward runs the operator's own backward kernels with the chain
+rule through the three lines applied inside the first of them -- gradients for value, reference points, offsets
+and logits; locations, weights and their gradients never reach memory either.
 """
 import torch
 from torch.amp import custom_bwd, custom_fwd
@@ -53,29 +53,19 @@ class MultiScaleDeformableAttnFusedFunction(Function):
         output = _C.msda_fused_forward(value, value_spatial_shapes, value_level_start_index, reference_points,
                                        sampling_offsets, attention_logits)
         ctx.save_for_backward(value, value_spatial_shapes, value_level_start_index, reference_points,
-                              sampling_offsets, attention_logits)
+                              sampling_offsets, attention_logits, output)
         return output
 
     @staticmethod
     @once_differentiable
     @custom_bwd(device_type="cuda")
     def backward(ctx, grad_output):
-        value, shapes, lsi, ref, off, logits = ctx.saved_tensors
+        value, shapes, lsi, ref, off, logits, output = ctx.saved_tensors
         need = ctx.needs_input_grad
-        with torch.enable_grad():
-            ref_g = ref.detach().requires_grad_(need[3])
-            off_g = off.detach().requires_grad_(need[4])
-            log_g = logits.detach().requires_grad_(need[5])
-            loc, attn = sampling_inputs(shapes, ref_g, off_g, log_g)
-        grad_value, grad_loc, grad_attn = _C.multi_scale_deformable_attn_backward(
-            value, shapes, lsi, loc.detach(), attn.detach(), grad_output)
-        wanted = [t for t, n in ((ref_g, need[3]), (off_g, need[4]), (log_g, need[5])) if n]
-        grads = iter(torch.autograd.grad([loc, attn], wanted, [grad_loc, grad_attn], allow_unused=True)
-                     if wanted else ())
-        g_ref = next(grads) if need[3] else None
-        g_off = next(grads) if need[4] else None
-        g_log = next(grads) if need[5] else None
-        return (grad_value if need[0] else None), None, None, g_ref, g_off, g_log
+        grad_value, g_ref, g_off, g_log = _C.msda_fused_backward(
+            value, shapes, lsi, ref, off, logits, output, grad_output, need_grad_reference_points=need[3])
+        return (grad_value if need[0] else None), None, None, g_ref, (g_off if need[4] else None), \
+            (g_log if need[5] else None)
 
 
 multi_scale_deformable_attn_fused = MultiScaleDeformableAttnFusedFunction.apply

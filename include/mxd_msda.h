@@ -131,6 +131,24 @@ int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, con
                            const void* attn_logits, void* output, int dtype, int64_t bs, int64_t nk, int64_t nh,
                            int64_t hd, int64_t nl, int64_t nq, int64_t np, void* hip_stream);
 
+/* Backward of mxd_msda_fused_forward: the operator's backward with the chain rule through the
+ * softmax and through the location arithmetic applied inside the first kernel, so that neither
+ * locations and weights nor their gradients reach memory.  `output` is the forward result (the
+ * softmax backward uses, per (query, head), the dot product of its row with the grad_output row).
+ * grad_sampling_offsets and grad_attn_logits have the shapes and dtype of their inputs and are
+ * fully overwritten; grad_value as in mxd_msda_backward (flags: MXD_BWD_ACCUMULATE).
+ * grad_reference_points [bs,nq,nl,ref_dim] may be NULL when the caller does not need it (the sum
+ * over heads then is skipped); pass the same choice (want_grad_ref 0/1) to the workspace query,
+ * which adds nh*bs*nq*nl*ref_dim floats of per-head partial sums to the operator's own scratch. */
+size_t mxd_msda_fused_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd,
+                                               int64_t nl, int64_t nq, int64_t np, int ref_dim, int want_grad_ref);
+int mxd_msda_fused_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                            const void* reference_points, int ref_dim, const void* sampling_offsets,
+                            const void* attn_logits, const void* output, const void* grad_output, void* grad_value,
+                            void* grad_reference_points, void* grad_sampling_offsets, void* grad_attn_logits,
+                            void* workspace, size_t workspace_bytes, int dtype, int64_t bs, int64_t nk, int64_t nh,
+                            int64_t hd, int64_t nl, int64_t nq, int64_t np, int flags, void* hip_stream);
+
 /* Bytes of scratch mxd_msda_backward needs (0 if the sizes are invalid, and for float32 sizes
  * that take the one-kernel path with global atomics).  It holds the hand-over between the two
  * backward kernels -- a table of run starts and two 16-byte records per sample, written

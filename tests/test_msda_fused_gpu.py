@@ -34,7 +34,7 @@ def make_fused_inputs(name, ref_dim=2, scale_queries=1.0, seed=77, dtype=torch.f
 
 def _edge_masks(shapes, ref, off, logits):
     """Samples whose float32 location lies within 2^-20 px of (not on) a cell edge -- the location gradient
-    jumps there -- and the reference points that own such a sample."""
+    jumps there -- or exactly on pixel coordinate -1, and the reference points that own such a sample."""
     loc = orc.fused_sampling_inputs(shapes, ref.float(), off.float(), logits.float())[0].double()
     near = torch.zeros(loc.shape[:-1], dtype=torch.bool)
     for lvl, (h, w) in enumerate(shapes.tolist()):
@@ -42,6 +42,9 @@ def _edge_masks(shapes, ref, off, logits):
         h_im = loc[:, :, :, lvl, :, 1] * h - 0.5
         dw, dh = (w_im - w_im.round()).abs(), (h_im - h_im.round()).abs()
         near[:, :, :, lvl] = ((dw > 0) & (dw < 2.0 ** -20)) | ((dh > 0) & (dh < 2.0 ** -20))
+        # a pixel coordinate of exactly -1 (16-bit inputs reach it): the operator drops the sample, as the
+        # reference's kernels do, where grid_sample still reports a location gradient from the weight-0 corner
+        near[:, :, :, lvl] |= (w_im == -1.0) | (h_im == -1.0)
     ref_near = near.any(dim=4).any(dim=2)                     # [bs, nq, nl]
     return near.numpy(), ref_near.numpy()
 
@@ -120,6 +123,65 @@ def test_fused_more_than_16_samples_per_unit_and_many_heads(gpu_device):
     _compare(got, want, shapes, ref, off, logits, (FWD_FP32,) + (BWD_FP32,) * 4)
 
 
+@pytest.mark.parametrize("npts,nl,ref_dim", [(3, 3, 2), (3, 2, 4), (32, 2, 2), (1, 5, 4)])
+def test_fused_gradients_other_point_counts(gpu_device, npts, nl, ref_dim):
+    """Point counts that are not a power of two, or exceed one staging chunk: the reference points' gradient is
+    then added up with atomics instead of across lanes."""
+    g = torch.Generator().manual_seed(100 + npts)
+    shapes, lsi = workloads.level_tensors(((12, 17), (6, 9), (3, 5), (2, 3), (1, 2))[:nl])
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh, hd = 2, 157, 3, 32
+    value = torch.randn(bs, nk, nh, hd, generator=g)
+    ref = torch.rand(bs, nq, nl, ref_dim, generator=g)
+    if ref_dim == 4:
+        ref[..., 2:] = ref[..., 2:] * 0.3 + 0.05
+    off = torch.randn(bs, nq, nh, nl, npts, 2, generator=g) * 2
+    logits = torch.randn(bs, nq, nh, nl * npts, generator=g) * 2
+    grad_out = torch.randn(bs, nq, nh * hd, generator=g)
+    want = orc.fused_fwd_bwd(value, shapes, ref, off, logits, grad_out, loc_dtype=torch.float32)
+    got = _run(value, shapes, lsi, ref, off, logits, grad_out, gpu_device)
+    _compare(got, want, shapes, ref, off, logits, (FWD_FP32,) + (BWD_FP32,) * 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ref_dim", [2, 4])
+def test_fused_gradients_16bit(gpu_device, dtype, ref_dim):
+    """Gradients in 16-bit storage: float64 oracle on the rounded inputs, locations formed in float32 as the
+    kernel forms them.  bfloat16 results carry one rounding of up to 2^-9 relative, which the error measure
+    (largest error over largest element) can see in full."""
+    inp = make_fused_inputs("tiny", ref_dim, 1.0, dtype=dtype)
+    value, shapes, lsi, ref, off, logits, grad_out = inp
+    want = orc.fused_fwd_bwd(value.double(), shapes, ref.double(), off.double(), logits.double(), grad_out.double(),
+                             loc_dtype=torch.float32)
+    got = _run(*inp, gpu_device)
+    tol = HALF if dtype == torch.float16 else 2.0 ** -8
+    # the logits' gradient takes the softmax backward's sum from the stored (rounded) forward result and is
+    # rounded itself: two roundings
+    _compare(got, want, shapes, ref, off, logits, (tol,) * 4 + (2 * tol,))
+
+
+def test_fused_backward_without_reference_point_gradient(gpu_device):
+    """Reference points that need no gradient: the per-head partial sums and their reduction are skipped and
+    the other gradients are unchanged."""
+    inp = make_fused_inputs("tiny", 2, 1.0)
+    value, shapes, lsi, ref, off, logits, grad_out = inp
+    full = _run(*inp, gpu_device)
+    v = value.to(gpu_device).requires_grad_()
+    o = off.to(gpu_device).requires_grad_()
+    z = logits.to(gpu_device).requires_grad_()
+    out = drivingsdk_amd.multi_scale_deformable_attn_fused(v, shapes.to(gpu_device), lsi.to(gpu_device),
+                                                           ref.to(gpu_device), o, z)
+    out.backward(grad_out.to(gpu_device))
+    for got, want in zip((out, o.grad, z.grad), (full[0], full[3], full[4])):
+        np.testing.assert_array_equal(got.detach().double().cpu().numpy(), want)
+    # (grad_value is summed in an order that varies from run to run)
+    assert rel_err(v.grad.double().cpu().numpy(), full[1]) <= 1e-6
+    lib = _lib.load()
+    with_ref = lib.mxd_msda_fused_backward_workspace_bytes(0, 1, 1360, 8, 32, 4, 1360, 4, 2, 1)
+    without = lib.mxd_msda_fused_backward_workspace_bytes(0, 1, 1360, 8, 32, 4, 1360, 4, 2, 0)
+    assert with_ref - without == 8 * 1360 * 4 * 2 * 4
+
+
 def test_fused_error_paths(gpu_device):
     inp = make_fused_inputs("tiny", 2, 0.05)
     value, shapes, lsi, ref, off, logits, _ = [t.to(gpu_device) for t in inp]
@@ -130,3 +192,5 @@ def test_fused_error_paths(gpu_device):
                                                          logits.cpu())
     lib = _lib.load()
     assert lib.mxd_msda_fused_forward(None, None, None, None, 2, None, None, None, 0, 1, 10, 1, 8, 1, 1, 1, None) == -3
+    assert lib.mxd_msda_fused_backward(*([None] * 4), 2, *([None] * 9), 0, 0, 1, 10, 1, 8, 1, 1, 1, 0, None) == -3
+    assert lib.mxd_msda_fused_backward_workspace_bytes(0, 1, 10, 1, 8, 1, 1, 1, 3, 1) == 0
