@@ -180,10 +180,25 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
 }
 
 // Bytes of LDS the plain forward sets aside for the rows of the last levels (0: none).  Needs 16-byte lanes.
-int forward_cache_bytes(int vec, int es)
+// LDS for the forward's level cache, 0 = run without.  The cache pays when the coarsest level fits in it
+// (a quarter of the samples of a 4-level pyramid then are gathered from LDS) and costs otherwise: its
+// workgroups are larger and hold more LDS, which leaves fewer wavefronts per CU.  The level shapes live in
+// device memory, so the decision here rests on an estimate: in a pyramid that halves from level to level
+// the last one has nk*3/(4^nl - 1) pixels.  With more than 8 units per wavefront (rows of 64 bytes) the
+// staging strips alone limit the wavefronts per CU, and the cache is left out.
+// MXD_MSDA_FWD_LDS set in the environment overrides the estimate (0 = off, bytes = on).
+int forward_cache_bytes(int vec, int es, const Dims& d, int units_per_wave)
 {
+    const char* forced = getenv("MXD_MSDA_FWD_LDS");
     const int v = env_int("MXD_MSDA_FWD_LDS", 32768);
-    return (vec * es == 16 && v >= 1024 && v <= 65536) ? (v & ~15) : 0;
+    if (!(vec * es == 16 && v >= 1024 && v <= 65536)) return 0;
+    if (!(forced && *forced)) {
+        if (units_per_wave > 8) return 0;
+        double last = (double)d.nk;
+        if (d.nl > 1) last = (double)d.nk * 3.0 / ((double)(int64_t(1) << (2 * (d.nl < 16 ? d.nl : 16))) - 1.0);
+        if (last * 1.1 * (double)(d.hd * es) > (double)v) return 0;
+    }
+    return v & ~15;
 }
 
 // level_cache: in/out, bytes of LDS for the forward's level cache (asked for -> granted)
@@ -211,7 +226,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     const BwdLayout L = bwd_layout(dtype, d);
     // the tile pass wants L.tile_q queries per workgroup of the first backward kernel
     if (backward) iters = L.tiles ? (int)(L.tile_q / (p->units_per_wave * p->waves_per_block)) : 1;
-    int cache = (level_cache && *level_cache && !backward) ? forward_cache_bytes(vec, es) : 0;
+    int cache = (level_cache && *level_cache && !backward) ? forward_cache_bytes(vec, es, d, p->units_per_wave) : 0;
     if (cache > 0) {
         // 8 wavefronts share one copy of the cached rows and work through 256 queries; two such workgroups
         // must fit a CU (80 KiB each), else fewer wavefronts, else no cache

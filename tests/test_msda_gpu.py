@@ -379,6 +379,20 @@ def test_backward_launch_variants_agree_with_the_oracle(gpu_device, monkeypatch,
         print(env, name, errs)
 
 
+@pytest.mark.parametrize("lds", ["0", "2048", "32768", "49152", "65536"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
+    """The forward's level cache (rows of the last levels held in LDS) is switched by an estimate of the level
+    sizes; here it is forced off and on with room for no, one, several and all levels, for every dtype."""
+    monkeypatch.setenv("MXD_MSDA_FWD_LDS", lds)
+    tol = FWD_FP32 if dtype == torch.float32 else (HALF if dtype == torch.float16 else 2.0 ** -8)
+    for name, scale in (("tiny", 1.0), ("detr_encoder", 0.1)):
+        inp = workloads.make_inputs(name, dtype=dtype, scale_queries=scale)
+        want = oracle_all(inp, with_grads=False)[0]
+        got = run_gpu(inp, gpu_device, with_grads=False)[0]
+        assert rel_err(got, want) <= tol, (name, lds, dtype)
+
+
 def _random_case(seed):
     """A random small problem: odd sizes everywhere, locations reaching outside the image."""
     rng = np.random.default_rng(seed)
