@@ -9,6 +9,9 @@ Deformable-DETR encoder shape (bs 2, 19947 queries = keys, 8 heads x 32, 4 level
 float32).  Prints ONE JSON line: whole-step throughput in queries/s, the HBM roofline of the
 dominant kernel (timed live with HIP events on the launch stream), per-kernel figures, and
 the CPU oracle timed on the host cores of the same box as a reported baseline.
+Other workloads: the named shapes of drivingsdk_amd.workloads (with --dtype), and the sibling operators
+that run on the same kernels: sparse4d_dagg (deformable aggregation), gka (geometric kernel attention),
+grid_sampler2d (grid_sampler2d_v2), each at a shape of the reference's recipes or tests.
 """
 import argparse
 import json
@@ -233,6 +236,122 @@ def _bench_dagg(args):
     print(json.dumps(result))
 
 
+def _op_result(args, metric, units, unit, ms_step, ms_fwd, b_fwd, b_bwd, workload):
+    return {"metric": metric, "value": units / (ms_step * 1e-3), "unit": unit, "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": workload},
+            "roofline": {"bound": "hbm", "kernel": "forward + backward kernels of one step",
+                         "achieved": (b_fwd + b_bwd) / (ms_step * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": (b_fwd + b_bwd) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                         "algorithmic_bytes": b_fwd + b_bwd, "kernel_ms": ms_step},
+            "kernels": {"forward_ms": ms_fwd, "forward_algorithmic_GBps": b_fwd / (ms_fwd * 1e-3) / 1e9}}
+
+
+def _bench_gka(args):
+    """Geometric kernel attention at the largest shape of the reference's test
+    (tests/torch/test_geometric_kernel_attention.py:112: bs 24, 7156 queries, 4 heads x 64, one 15x25 level, 15 points,
+    pixel-index locations reaching 3 px outside the map): forward + backward through the autograd Function."""
+    import torch
+
+    import mx_driving
+    from oracle import gka_oracle
+
+    dev = torch.device("cuda", 0)
+    bs, nq, hd, nh, nl, npts, (H, W) = 24, 7156, 64, 4, 1, 15, (15, 25)
+    g = torch.Generator().manual_seed(2025)
+    sh = torch.tensor([[H, W]] * nl)
+    lsi = torch.cat((sh.new_zeros((1,)), sh.prod(1).cumsum(0)[:-1]))
+    nk = int(sh.prod(1).sum())
+    loc = torch.rand(bs, nq, nh, nl, npts, 2, generator=g)
+    loc[..., 0] = loc[..., 0] * (W + 6) - 3
+    loc[..., 1] = loc[..., 1] * (H + 6) - 3
+    loc = loc.long().float()
+    value_c = torch.rand(bs, nk, nh, hd, generator=g) * 3
+    attn_c = torch.rand(bs, nq, nh, nl, npts, generator=g)
+    go_c = torch.rand(bs, nq, nh * hd, generator=g) * 10
+    value, attn = value_c.to(dev).requires_grad_(), attn_c.to(dev).requires_grad_()
+    locd, go, shd, lsid = loc.to(dev), go_c.to(dev), sh.int().to(dev), lsi.int().to(dev)
+
+    def step():
+        value.grad = attn.grad = None
+        mx_driving.geometric_kernel_attention(value, shd, lsid, locd, attn).backward(go)
+
+    def fwd():
+        with torch.no_grad():
+            mx_driving.geometric_kernel_attention(value, shd, lsid, locd, attn)
+
+    ms_step = _event_ms(step, args.steps, args.warmup)
+    ms_fwd = _event_ms(fwd, args.steps, args.warmup)
+    # every tensor once: value, locations, weights in, output out; backward: the same inputs + grad_output in,
+    # grad_value and grad_attn_weights out
+    b_fwd = 4 * (value.numel() + loc.numel() + attn.numel() + go.numel())
+    b_bwd = 4 * (value.numel() + loc.numel() + attn.numel() + go.numel() + value.numel() + attn.numel())
+    result = _op_result(args, "geometric_kernel_attention fwd+bwd queries/s, reference test shape", bs * nq, "queries/s",
+                        ms_step, ms_fwd, b_fwd, b_bwd,
+                        f"gka: bs={bs}, queries={nq}, keys={nk} ({H}x{W}), heads={nh}x{hd}, levels={nl}, points={npts}")
+    if not args.no_cpu_baseline:
+        n = 2  # batch elements timed on the CPU
+        t0 = time.perf_counter()
+        part = (value_c[:n], sh, lsi, loc[:n], attn_c[:n])
+        gka_oracle.forward(*part)
+        gka_oracle.backward(*part, go_c[:n])
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": n * nq / dt, "unit": "queries/s", "cores": 1, "kind": "port",
+                                  "sample": f"{n} of the {bs} batch elements, forward + backward of the numpy restatement"}
+    print(json.dumps(result))
+
+
+def _bench_grid_sampler(args):
+    """grid_sampler2d_v2 at the largest shape of the reference's test (tests/torch/test_grid_sampler2d_v2.py:59: input
+    [24, 128, 64, 176], grid [24, 24, 176, 2], bilinear, zeros padding, align_corners False): forward + backward."""
+    import torch
+    import torch.nn.functional as F
+
+    import mx_driving
+
+    dev = torch.device("cuda", 0)
+    n, c, h, w, ho, wo = 24, 128, 64, 176, 24, 176
+    g = torch.Generator().manual_seed(2026)
+    x_c = torch.rand(n, c, h, w, generator=g)
+    grid_c = 2 * torch.rand(n, ho, wo, 2, generator=g) - 1
+    go_c = torch.randn(n, c, ho, wo, generator=g)
+    # the operator works on channel-last memory; give it channel-last tensors as a channel-last model would, so that
+    # the step holds the sampler's kernels and no layout copies
+    x = x_c.to(dev).contiguous(memory_format=torch.channels_last).requires_grad_()
+    grid = grid_c.to(dev).requires_grad_()
+    go = go_c.to(dev).contiguous(memory_format=torch.channels_last)
+
+    def step():
+        x.grad = grid.grad = None
+        mx_driving.grid_sampler2d_v2(x, grid, "bilinear", "zeros", False).backward(go)
+
+    def fwd():
+        with torch.no_grad():
+            mx_driving.grid_sampler2d_v2(x, grid, "bilinear", "zeros", False)
+
+    ms_step = _event_ms(step, args.steps, args.warmup)
+    ms_fwd = _event_ms(fwd, args.steps, args.warmup)
+    b_fwd = 4 * (x.numel() + grid.numel() + go.numel())
+    b_bwd = 4 * (x.numel() + grid.numel() + go.numel() + x.numel() + grid.numel())
+    result = _op_result(args, "grid_sampler2d_v2 fwd+bwd output pixels/s, reference test shape", n * ho * wo, "pixels/s",
+                        ms_step, ms_fwd, b_fwd, b_bwd,
+                        f"grid_sampler2d: input=[{n},{c},{h},{w}], grid=[{n},{ho},{wo},2], bilinear, zeros, "
+                        "align_corners=False, channel-last tensors")
+    if not args.no_cpu_baseline:
+        xr, gr = x_c.clone().requires_grad_(), grid_c.clone().requires_grad_()
+        times = []
+        for _ in range(4):
+            xr.grad = gr.grad = None
+            t0 = time.perf_counter()
+            F.grid_sample(xr, gr, "bilinear", "zeros", False).backward(go_c)
+            times.append(time.perf_counter() - t0)
+        dt = sorted(times[1:])[1]
+        result["cpu_baseline"] = {"value": n * ho * wo / dt, "unit": "pixels/s", "cores": torch.get_num_threads(),
+                                  "kind": "port", "sample": "3 timed forward+backward iterations (median) of torch's "
+                                  "grid_sample on the CPU in float32, the golden of the reference's test"}
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -260,6 +379,10 @@ def main():
     _lib.load()
     if args.workload == "sparse4d_dagg":
         return _bench_dagg(args)
+    if args.workload == "gka":
+        return _bench_gka(args)
+    if args.workload == "grid_sampler2d":
+        return _bench_grid_sampler(args)
     dev = torch.device("cuda", 0)
     dtype = getattr(torch, args.dtype)
     inp = workloads.make_inputs(args.workload, dtype=dtype, with_grad_output=True)

@@ -375,7 +375,9 @@ def geometric_kernel_attention_backward(value, spatial_shapes, level_start_index
 
 def grid_sampler2d_v2(input, grid, interpolation_mode, padding_mode, align_corners):
     """input [N, C, H, W], grid [N, H_out, W_out, 2] -> output [N, C, H_out, W_out] (bilinear).  As in the reference's
-    binding the kernel works on channel-last data: input is permuted to NHWC before and the output back after."""
+    binding the kernel works on channel-last data: input is permuted to NHWC before and the output back after.
+    An input in torch's channels_last memory format needs no copy and gets its output in that format too (torch's
+    convention for memory formats); any other input gets a contiguous NCHW output as in the reference."""
     _check(input.layout == torch.strided and grid.layout == torch.strided,
            "grid_sampler2d_v2(): expected input and grid to have torch.strided layout")
     _check(input.dtype in _FLOAT_CODES and grid.dtype == input.dtype,
@@ -403,7 +405,8 @@ def grid_sampler2d_v2(input, grid, interpolation_mode, padding_mode, align_corne
                                             w_in, h_out, w_out, int(interpolation_mode), int(padding_mode),
                                             int(bool(align_corners)), torch.cuda.current_stream().cuda_stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
-    return out.permute(0, 3, 1, 2).contiguous()
+    channels_last = input.is_contiguous(memory_format=torch.channels_last) and not input.is_contiguous()
+    return out.permute(0, 3, 1, 2) if channels_last else out.permute(0, 3, 1, 2).contiguous()
 
 
 def grid_sampler2d_v2_backward(grad_output, input_x, input_grid, interpolation_mode, padding_mode, align_corners):

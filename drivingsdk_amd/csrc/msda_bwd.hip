@@ -37,6 +37,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
     constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
     constexpr bool FUSED = SRC == kSrcFused;
+    constexpr int NC = SRC == kSrcGka ? 1 : 4;  // corner rows per sample (geometric kernel attention: one pixel)
 
     extern __shared__ __align__(16) unsigned char smem[];
     i32x4* lvl = reinterpret_cast<i32x4*>(smem);
@@ -260,20 +261,20 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     float d[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int p = 0; p < NPASS; ++p) {
-                        typename RowIO<T, VEC>::raw_t raw[4];
+                        typename RowIO<T, VEC>::raw_t raw[NC];
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
+                        for (int k = 0; k < NC; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
 #pragma unroll
-                        for (int k = 0; k < 4; ++k) {
+                        for (int k = 0; k < NC; ++k) {
                             float v[VEC];
                             RowIO<T, VEC>::unpack(raw[k], v);
 #pragma unroll
                             for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
                         }
                     }
-                    f32x4 dsum;
+                    f32x4 dsum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) dsum[k] = group_sum<LG>(d[k]);
+                    for (int k = 0; k < NC; ++k) dsum[k] = group_sum<LG>(d[k]);
                     if (c == 0) dots[g * kChunk + sl] = dsum;
                 }
             };

@@ -41,6 +41,7 @@ template <typename T, int VEC, int NPASS, int SRC, bool LDSC>
 __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs a)
 {
     constexpr bool FUSED = SRC == kSrcFused;
+    constexpr int NC = SRC == kSrcGka ? 1 : 4;  // corner rows per sample (geometric kernel attention: one pixel)
     static_assert(!LDSC || (SRC == kSrcPlain && VEC * sizeof(T) == 16), "the level cache is built for 16-byte lanes");
     extern __shared__ __align__(16) unsigned char smem[];
     i32x4* lvl = reinterpret_cast<i32x4*>(smem);                               // [kMaxLevels]
@@ -213,11 +214,11 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
                 const f32x4 w = *reinterpret_cast<const f32x4*>(mine[sl].w);
 #pragma unroll
                 for (int p = 0; p < NPASS; ++p) {
-                    typename RowIO<T, VEC>::raw_t raw[4];
+                    typename RowIO<T, VEC>::raw_t raw[NC];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
+                    for (int k = 0; k < NC; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
+                    for (int k = 0; k < NC; ++k) {
                         float v[VEC];
                         RowIO<T, VEC>::unpack(raw[k], v);
 #pragma unroll

@@ -98,3 +98,19 @@ def test_unsupported_modes_go_to_torch_and_errors(gpu_device):
     assert lib.mxd_grid_sampler2d_forward(None, None, None, 0, 1, 4, 6, 6, 3, 3, 0, 0, 0, None) == -3
     assert lib.mxd_grid_sampler2d_forward(None, None, None, 0, 1, 4, 6, 6, 3, 3, 1, 0, 0, None) == -2
     assert lib.mxd_grid_sampler2d_forward(None, None, None, 0, 1, 4, 6, 6, 3, 3, 0, 2, 0, None) == -2
+
+
+def test_channels_last_input_keeps_its_memory_format(gpu_device):
+    """A channels_last input is used in place (it is the layout the kernel works on) and the output comes back
+    in the same memory format, with the same values as for a contiguous input."""
+    x, grid, go = make_inputs([3, 32, 20, 30], [3, 11, 17, 2], seed=9, span=1.1)
+    xd, gd = x.to(gpu_device), grid.to(gpu_device)
+    plain = mx_driving.grid_sampler2d_v2(xd, gd, "bilinear", "zeros", False)
+    xcl = xd.contiguous(memory_format=torch.channels_last).requires_grad_()
+    out = mx_driving.grid_sampler2d_v2(xcl, gd, "bilinear", "zeros", False)
+    assert plain.is_contiguous() and out.is_contiguous(memory_format=torch.channels_last) and not out.is_contiguous()
+    assert torch.equal(out, plain)
+    out.backward(go.to(gpu_device).contiguous(memory_format=torch.channels_last))
+    xr = x.double().requires_grad_()
+    F.grid_sample(xr, grid.double(), "bilinear", "zeros", False).backward(go.double())
+    assert rel_err(xcl.grad.double().cpu().numpy(), xr.grad.numpy()) <= BWD_FP32
