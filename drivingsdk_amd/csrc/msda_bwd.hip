@@ -218,7 +218,18 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 
         for (int c0 = 0; c0 < a.S; c0 += kChunk) {
             // ---- geometry -----------------------------------------------------------------
-            for (int i = lane; i < entries; i += kWave) {
+            // A lane stages entries/64 <= kLaneSamples samples per pass and meets the same samples again when
+            // their dots are reduced: for the first kKeep of them (all, with up to 8 units per wavefront)
+            // fractions, weight, first pixel and validity bits stay in registers until then instead of being
+            // derived from the location a second time.
+            constexpr int kLaneSamples = 4, kKeep = 2;
+            float keep_lw[kKeep], keep_lh[kKeep], keep_aw[kKeep], keep_wf[kKeep], keep_hf[kKeep];
+            int32_t keep_pix[kKeep];
+            uint32_t keep_fl[kKeep];  // bit 0 valid, bits 1..4 corner valid, bits 8.. level
+#pragma unroll
+            for (int ks = 0; ks < kLaneSamples; ++ks) {
+                const int i = lane + ks * kWave;
+                if (i >= entries) break;
                 const int u = i >> 4, sl = i & (kChunk - 1);
                 const int s = c0 + sl, q = q0 + u;
                 const bool active = (q < wk.q_end) && (s < a.S);
@@ -245,6 +256,16 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
                 }
                 stage[u * kChunkStride + sl] = en;
+                if (ks < kKeep) {
+                    keep_lw[ks % kKeep] = sm.lw;
+                    keep_lh[ks % kKeep] = sm.lh;
+                    keep_aw[ks % kKeep] = aw;
+                    keep_wf[ks % kKeep] = sm.Wf;
+                    keep_hf[ks % kKeep] = sm.Hf;
+                    keep_pix[ks % kKeep] = sm.pix[0];
+                    keep_fl[ks % kKeep] = (sm.valid ? 1u : 0u) | (sm.cvalid[0] ? 2u : 0u) | (sm.cvalid[1] ? 4u : 0u) |
+                                          (sm.cvalid[2] ? 8u : 0u) | (sm.cvalid[3] ? 16u : 0u) | ((uint32_t)l << 8);
+                }
             }
             wave_lds_sync();
 
@@ -318,25 +339,55 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             }
 
             // ---- grad_attn / grad_loc from the reduced dots, one sample per lane ----------
-            for (int i = lane; i < entries; i += kWave) {
+#pragma unroll
+            for (int ks = 0; ks < kLaneSamples; ++ks) {
+                const int i = lane + ks * kWave;
+                if (i >= entries) break;
                 const int u = i >> 4, sl = i & (kChunk - 1);
                 const int s = c0 + sl, q = q0 + u;
                 if ((q < wk.q_end) && (s < a.S)) {
                     const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
-                    float x = to_f32(loc[2 * sr.loc_e]);
-                    float y = to_f32(loc[2 * sr.loc_e + 1]);
-                    float aw = 1.0f;
-                    if constexpr (SRC != kSrcGrid) aw = to_f32(attn[sr.w_e]);
-                    const int l = sr.l;
-                    const float ox = x, oy = y;  // raw offsets (fused form)
-                    const T* rp = nullptr;
-                    if constexpr (FUSED) {
-                        rp = ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim;
-                        fused_location(a, rp, lvl[l], x, y);
-                        aw = expf(aw - unit_stats(u)[0]) / unit_stats(u)[1];
+                    int l = sr.l;
+                    float aw = 1.0f, ox = 0.f, oy = 0.f;  // (ox, oy): raw offsets of the fused form
+                    Sample sm;
+                    if (ks < kKeep) {
+                        // the sample as the geometry pass left it
+                        const uint32_t fl = keep_fl[ks % kKeep];
+                        l = (int)(fl >> 8);
+                        aw = keep_aw[ks % kKeep];
+                        sm.valid = (fl & 1u) != 0;
+                        sm.lw = keep_lw[ks % kKeep];
+                        sm.lh = keep_lh[ks % kKeep];
+                        sm.Wf = keep_wf[ks % kKeep];
+                        sm.Hf = keep_hf[ks % kKeep];
+                        float wt[4];
+                        bilinear_weights(sm.lw, sm.lh, wt);
+                        const int32_t Wl = lvl[l].y;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            sm.pix[k] = keep_pix[ks % kKeep] + (k & 1) + (k >> 1) * Wl;
+                            sm.cvalid[k] = ((fl >> (1 + k)) & 1u) != 0;
+                            sm.w[k] = sm.valid ? wt[k] : 0.0f;
+                        }
+                        if constexpr (FUSED) {
+                            ox = to_f32(loc[2 * sr.loc_e]);
+                            oy = to_f32(loc[2 * sr.loc_e + 1]);
+                        }
+                    } else {
+                        float x = to_f32(loc[2 * sr.loc_e]);
+                        float y = to_f32(loc[2 * sr.loc_e + 1]);
+                        if constexpr (SRC != kSrcGrid) aw = to_f32(attn[sr.w_e]);
+                        ox = x;
+                        oy = y;
+                        if constexpr (FUSED) {
+                            fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim, lvl[l], x, y);
+                            aw = expf(aw - unit_stats(u)[0]) / unit_stats(u)[1];
+                        }
+                        const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
+                        sm = source_geometry<SRC>(x, y, lvl[l], a.nk, inside, a.grid);
                     }
-                    const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                    const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, inside, a.grid);
+                    const T* rp = nullptr;
+                    if constexpr (FUSED) rp = ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim;
                     const f32x4 dd = dots[u * kChunk + sl];
                     float ga = 0.f, gx = 0.f, gy = 0.f;
                     if (sm.valid) {

@@ -261,6 +261,17 @@ struct Sample {
     bool valid;      // sample lies inside (-1, W) x (-1, H) in pixel space; false for NaN/Inf
 };
 
+// Bilinear corner weights from the fractions, in the corner order of Sample.
+__device__ inline void bilinear_weights(float lw, float lh, float (&w)[4])
+{
+#pragma clang fp contract(off)
+    const float hw = 1.0f - lw, hh = 1.0f - lh;
+    w[0] = hh * hw;
+    w[1] = hh * lw;
+    w[2] = lh * hw;
+    w[3] = lh * lw;
+}
+
 // level = {H, W, level_start_index, unused}
 __device__ inline Sample sample_geometry(float x, float y, i32x4 level, int32_t nk, bool active)
 {
@@ -299,7 +310,8 @@ __device__ inline Sample sample_geometry(float x, float y, i32x4 level, int32_t 
     s.pix[2] = p00 + W;
     s.pix[3] = p00 + W + 1;
     const bool cv[4] = {vy0 && vx0, vy0 && vx1, vy1 && vx0, vy1 && vx1};
-    const float wt[4] = {hh * hw, hh * s.lw, s.lh * hw, s.lh * s.lw};
+    float wt[4];
+    bilinear_weights(s.lw, s.lh, wt);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         s.cvalid[k] = s.valid && cv[k] && ((uint32_t)s.pix[k] < (uint32_t)nk);
@@ -375,7 +387,8 @@ __device__ inline Sample grid_geometry(float gx, float gy, i32x4 level, int32_t 
     s.pix[2] = p00 + W;
     s.pix[3] = p00 + W + 1;
     const bool cv[4] = {vy0 && vx0, vy0 && vx1, vy1 && vx0, vy1 && vx1};
-    const float wt[4] = {hh * hw, hh * s.lw, s.lh * hw, s.lh * s.lw};
+    float wt[4];
+    bilinear_weights(s.lw, s.lh, wt);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         s.cvalid[k] = s.valid && cv[k] && ((uint32_t)s.pix[k] < (uint32_t)nk);
