@@ -184,3 +184,23 @@ def test_algorithmic_bytes_match_the_published_table():
     assert abs(mb("head_dim_128", torch.float16) - 97.02) < 0.01
     assert abs(mb("bevformer_sca") - 427.16) < 0.01
     assert abs(mb("bevformer_sca", torch.float16) - 213.58) < 0.01
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This build runs on one GPU: bench.py --gpus N (N > 1) says so and exits before touching a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_fused_backward_workspace_adds_the_reference_point_partials():
+    lib = _lib.load()
+    args = (0, 2, 19947, 8, 32, 4, 19947, 4)
+    plain = lib.mxd_msda_backward_workspace_bytes(0, 2, 19947, 8, 32, 4, 4, 19947, 4)
+    assert lib.mxd_msda_fused_backward_workspace_bytes(*args, 2, 0) == plain
+    assert lib.mxd_msda_fused_backward_workspace_bytes(*args, 2, 1) == plain + 8 * 2 * 19947 * 4 * 2 * 4
+    assert lib.mxd_msda_fused_backward_workspace_bytes(*args, 4, 1) == plain + 8 * 2 * 19947 * 4 * 4 * 4
+    assert lib.mxd_msda_fused_backward_workspace_bytes(*args, 3, 1) == 0
