@@ -282,6 +282,48 @@ def test_runs_on_a_side_stream_and_is_repeatable(gpu_device):
         assert rel_err(gv.double().cpu().numpy(), ref[1]) <= BWD_FP32  # atomics: order-dependent rounding only
 
 
+def test_forward_and_backward_replay_in_a_hip_graph(gpu_device):
+    """The launches of one forward + backward (zero-fill kernel, both backward kernels; no memset nodes) captured
+    in a HIP graph: three replays with fresh inputs copied into the captured tensors, the program's own eager
+    work and synchronisations between them, each replay compared with the eager result for the same inputs."""
+    from drivingsdk_amd import _C
+    base = workloads.make_inputs("detr_encoder_bwd", with_grad_output=True, scale_queries=0.05)
+    d = to_device(base, gpu_device)
+    sh, lsi = d.spatial_shapes.int(), d.level_start_index.int()
+    static = [t.clone() for t in (d.value, d.sampling_locations, d.attention_weights, d.grad_output)]
+
+    def run(v, lo, at, go):
+        out = _C.multi_scale_deformable_attn(v, sh, lsi, lo, at)
+        return (out,) + tuple(_C.multi_scale_deformable_attn_backward(v, sh, lsi, lo, at, go))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            run(*static)  # warm-up outside the capture (first-use set-up of the kernels)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run(*static)
+    g = torch.Generator().manual_seed(31)
+    for rep in range(3):
+        fresh = [torch.randn(t.shape, generator=g) * 0.5 for t in static]
+        fresh[1] = torch.rand(static[1].shape, generator=g) * 1.2 - 0.1
+        fresh[2] = torch.rand(static[2].shape, generator=g)
+        for dst, src in zip(static, fresh):
+            dst.copy_(src.to(gpu_device))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        eager = run(*[t.clone() for t in static])       # eager work between the replays
+        torch.cuda.synchronize()
+        for name, a_, b_, tol in zip(("output", "grad_value", "grad_loc", "grad_attn"), got, eager,
+                                     (0.0, 1e-6, 0.0, 0.0)):
+            err = rel_err(a_.double().cpu().numpy(), b_.double().cpu().numpy())
+            assert err <= tol, (rep, name, err)   # (grad_value: summation order varies from run to run)
+
+
 def test_linearity_at_full_size(gpu_device):
     """Size-independent property at the benchmark shape: linear in value and in the weights."""
     import mx_driving
@@ -391,6 +433,20 @@ def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
         want = oracle_all(inp, with_grads=False)[0]
         got = run_gpu(inp, gpu_device, with_grads=False)[0]
         assert rel_err(got, want) <= tol, (name, lds, dtype)
+
+
+def test_beyond_the_reference_limits(gpu_device):
+    """The reference refuses num_levels * num_points > 64; here 100 samples per (query, head) -- seven staging
+    passes, the last one partly filled -- at the largest head_dim (256), forward and gradients."""
+    g = torch.Generator().manual_seed(64)
+    shapes, lsi = workloads.level_tensors(((9, 14), (7, 5), (4, 6), (3, 3), (2, 2)))
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh, hd, nl, npts = 2, 77, 3, 256, 5, 20
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g), shapes, lsi,
+                               torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.2 - 0.1,
+                               torch.rand(bs, nq, nh, nl, npts, generator=g),
+                               torch.randn(bs, nq, nh * hd, generator=g))
+    print(_check_all(inp, gpu_device, FWD_FP32, BWD_FP32))
 
 
 def _random_case(seed):
