@@ -160,6 +160,10 @@ __device__ inline T from_f32(float v)
 template <typename T>
 __device__ inline void fused_location(const KArgs& a, const T* rp, const i32x4 lv, float& x, float& y)
 {
+    // every operation rounded on its own, wherever this is inlined: the backward derives the location of a
+    // sample in several places (counting records, staging, gradients) and all of them must land on the same
+    // pixel, as must the forward
+#pragma clang fp contract(off)
     if (a.ref_dim == 2) {
         x = to_f32(rp[0]) + x / (float)lv.y;
         y = to_f32(rp[1]) + y / (float)lv.x;
