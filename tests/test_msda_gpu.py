@@ -449,6 +449,41 @@ def test_beyond_the_reference_limits(gpu_device):
     print(_check_all(inp, gpu_device, FWD_FP32, BWD_FP32))
 
 
+def test_reference_onnx_export_shape(gpu_device):
+    """The shape of the reference's ONNX export test (tests/onnx/test_wrapper_onnx_ops.py:57-65): five large levels
+    whose sizes do not decrease (nk = 114400, 229 tiles per (batch, head)), 10000 queries; batch 2 of its 6."""
+    g = torch.Generator().manual_seed(114400)
+    shapes, lsi = workloads.level_tensors(((160, 140), (130, 120), (160, 240), (130, 120), (160, 140)))
+    assert lsi.tolist() == [0, 22400, 38000, 76400, 92000]
+    bs, nq, nh, hd, nl, npts = 2, 10000, 8, 32, 5, 4
+    inp = workloads.MsdaInputs(torch.rand(bs, 114400, nh, hd, generator=g), shapes, lsi,
+                               torch.rand(bs, nq, nh, nl, npts, 2, generator=g),
+                               torch.rand(bs, nq, nh, nl, npts, generator=g),
+                               torch.randn(bs, nq, nh * hd, generator=g))
+    print(_check_all(inp, gpu_device, FWD_FP32, BWD_FP32))
+
+
+@pytest.mark.parametrize("nq", [16, 3000])
+def test_documentation_example_all_samples_in_one_pixel(gpu_device, nq):
+    """The call example of the reference's documentation (docs/zh/api/context/multi_scale_deformable_attn.md:35-54):
+    one 100x100 level and every sampling location equal to 0.005, so all samples of a head fall into the same cell;
+    also with many queries, where one pixel list of the tile pass holds every record."""
+    g = torch.Generator().manual_seed(5)
+    shapes, lsi = workloads.level_tensors(((100, 100),))
+    bs, nh, hd, nl, npts = 1, 4, 32, 1, 8
+    inp = workloads.MsdaInputs(torch.rand(bs, 10000, nh, hd, generator=g) * 0.01, shapes, lsi,
+                               torch.ones(bs, nq, nh, nl, npts, 2) * 0.005,
+                               torch.rand(bs, nq, nh, nl, npts, generator=g) + 1e-5,
+                               torch.ones(bs, nq, nh * hd))
+    # 0.005 * 100 - 0.5 is pixel coordinate 0 to within rounding: every sample sits on a cell edge, where the
+    # location gradient jumps, so that gradient is only checked for being finite
+    want = oracle_all(inp)
+    got = run_gpu(inp, gpu_device)
+    for k, tol in ((0, FWD_FP32), (1, BWD_FP32), (3, BWD_FP32)):
+        assert rel_err(got[k], want[k]) <= tol, k
+    assert np.all(np.isfinite(got[2]))
+
+
 def _random_case(seed):
     """A random small problem: odd sizes everywhere, locations reaching outside the image."""
     rng = np.random.default_rng(seed)
