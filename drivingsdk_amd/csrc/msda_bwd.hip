@@ -222,11 +222,14 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             // their dots are reduced: for the first kKeep of them (all, with up to 8 units per wavefront)
             // fractions, weight, first pixel and validity bits stay in registers until then instead of being
             // derived from the location a second time.
-            constexpr int kLaneSamples = 4, kKeep = 2;
-            float keep_lw[kKeep], keep_lh[kKeep], keep_aw[kKeep], keep_wf[kKeep], keep_hf[kKeep];
-            int32_t keep_pix[kKeep];
-            uint32_t keep_fl[kKeep];  // bit 0 valid, bits 1..4 corner valid, bits 8.. level
-#pragma unroll
+            // (Only for the plain operator: the other sample sources run with fewer registers and more
+            // wavefronts per SIMD without it, which is worth more to them.)
+            constexpr int kLaneSamples = 4, kKeep = SRC == kSrcPlain ? 2 : 0, kKeepRegs = kKeep > 0 ? kKeep : 1;
+            float keep_lw[kKeepRegs], keep_lh[kKeepRegs], keep_aw[kKeepRegs], keep_wf[kKeepRegs], keep_hf[kKeepRegs];
+            int32_t keep_pix[kKeepRegs];
+            uint32_t keep_fl[kKeepRegs];  // bit 0 valid, bits 1..4 corner valid, bits 8.. level
+            constexpr int kUnroll = kKeep > 0 ? kLaneSamples : 1;  // (registers are indexed by ks: unrolled)
+#pragma unroll kUnroll
             for (int ks = 0; ks < kLaneSamples; ++ks) {
                 const int i = lane + ks * kWave;
                 if (i >= entries) break;
@@ -257,13 +260,13 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 }
                 stage[u * kChunkStride + sl] = en;
                 if (ks < kKeep) {
-                    keep_lw[ks % kKeep] = sm.lw;
-                    keep_lh[ks % kKeep] = sm.lh;
-                    keep_aw[ks % kKeep] = aw;
-                    keep_wf[ks % kKeep] = sm.Wf;
-                    keep_hf[ks % kKeep] = sm.Hf;
-                    keep_pix[ks % kKeep] = sm.pix[0];
-                    keep_fl[ks % kKeep] = (sm.valid ? 1u : 0u) | (sm.cvalid[0] ? 2u : 0u) | (sm.cvalid[1] ? 4u : 0u) |
+                    keep_lw[ks % kKeepRegs] = sm.lw;
+                    keep_lh[ks % kKeepRegs] = sm.lh;
+                    keep_aw[ks % kKeepRegs] = aw;
+                    keep_wf[ks % kKeepRegs] = sm.Wf;
+                    keep_hf[ks % kKeepRegs] = sm.Hf;
+                    keep_pix[ks % kKeepRegs] = sm.pix[0];
+                    keep_fl[ks % kKeepRegs] = (sm.valid ? 1u : 0u) | (sm.cvalid[0] ? 2u : 0u) | (sm.cvalid[1] ? 4u : 0u) |
                                           (sm.cvalid[2] ? 8u : 0u) | (sm.cvalid[3] ? 16u : 0u) | ((uint32_t)l << 8);
                 }
             }
@@ -276,7 +279,6 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             // uniform branches keep the row loads of the next samples from being issued early)
             auto gather_dots = [&](auto lg) {
                 constexpr int LG = decltype(lg)::value;
-#pragma unroll 2
                 for (int sl = 0; sl < ns; ++sl) {
                     const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
                     float d[4] = {0.f, 0.f, 0.f, 0.f};
@@ -339,7 +341,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             }
 
             // ---- grad_attn / grad_loc from the reduced dots, one sample per lane ----------
-#pragma unroll
+#pragma unroll kUnroll
             for (int ks = 0; ks < kLaneSamples; ++ks) {
                 const int i = lane + ks * kWave;
                 if (i >= entries) break;
@@ -352,20 +354,20 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     Sample sm;
                     if (ks < kKeep) {
                         // the sample as the geometry pass left it
-                        const uint32_t fl = keep_fl[ks % kKeep];
+                        const uint32_t fl = keep_fl[ks % kKeepRegs];
                         l = (int)(fl >> 8);
-                        aw = keep_aw[ks % kKeep];
+                        aw = keep_aw[ks % kKeepRegs];
                         sm.valid = (fl & 1u) != 0;
-                        sm.lw = keep_lw[ks % kKeep];
-                        sm.lh = keep_lh[ks % kKeep];
-                        sm.Wf = keep_wf[ks % kKeep];
-                        sm.Hf = keep_hf[ks % kKeep];
+                        sm.lw = keep_lw[ks % kKeepRegs];
+                        sm.lh = keep_lh[ks % kKeepRegs];
+                        sm.Wf = keep_wf[ks % kKeepRegs];
+                        sm.Hf = keep_hf[ks % kKeepRegs];
                         float wt[4];
                         bilinear_weights(sm.lw, sm.lh, wt);
                         const int32_t Wl = lvl[l].y;
 #pragma unroll
                         for (int k = 0; k < 4; ++k) {
-                            sm.pix[k] = keep_pix[ks % kKeep] + (k & 1) + (k >> 1) * Wl;
+                            sm.pix[k] = keep_pix[ks % kKeepRegs] + (k & 1) + (k >> 1) * Wl;
                             sm.cvalid[k] = ((fl >> (1 + k)) & 1u) != 0;
                             sm.w[k] = sm.valid ? wt[k] : 0.0f;
                         }

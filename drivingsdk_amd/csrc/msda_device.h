@@ -303,7 +303,6 @@ __device__ inline Sample sample_geometry(float x, float y, i32x4 level, int32_t 
     if (s.lh >= 1.0f) { fy += 1.0f; s.lh -= 1.0f; }
     const int32_t x0 = s.valid ? (int32_t)fx : 0;
     const int32_t y0 = s.valid ? (int32_t)fy : 0;
-    const float hw = 1.0f - s.lw, hh = 1.0f - s.lh;
     // two-sided (unsigned) tests: after the fraction fix-up a cell index may sit one step
     // outside [-1, size-1] for coordinates within an ulp of a validity edge
     const bool vx0 = (uint32_t)x0 < (uint32_t)W, vx1 = (uint32_t)(x0 + 1) < (uint32_t)W;
@@ -382,7 +381,6 @@ __device__ inline Sample grid_geometry(float gx, float gy, i32x4 level, int32_t 
     s.lw = ix - fx;
     s.lh = iy - fy;
     const int32_t x0 = s.valid ? (int32_t)fx : 0, y0 = s.valid ? (int32_t)fy : 0;
-    const float hw = 1.0f - s.lw, hh = 1.0f - s.lh;
     const bool vx0 = (uint32_t)x0 < (uint32_t)W, vx1 = (uint32_t)(x0 + 1) < (uint32_t)W;
     const bool vy0 = (uint32_t)y0 < (uint32_t)H, vy1 = (uint32_t)(y0 + 1) < (uint32_t)H;
     const int32_t p00 = base + y0 * W + x0;
