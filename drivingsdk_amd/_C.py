@@ -22,14 +22,20 @@ def _check(cond, msg):
         raise RuntimeError(msg)
 
 
+def _meta_flag(shapes):
+    """The reference's Python layer casts the level metadata to int32 on every call; int64 tensors are handed to the
+    library as they are instead (it reads the low words), which saves the two cast kernels."""
+    return _lib.META_I64 if shapes.dtype == torch.int64 else 0
+
+
 def _check_common(value, value_spatial_shapes, value_level_start_index, sampling_locations, attention_weights):
     _check(value.dtype in _FLOAT_CODES,
            f"value: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {value.dtype}")
-    _check(value_spatial_shapes.dtype == torch.int32,
-           f"value_spatial_shapes: int32 tensor expected but got a tensor with dtype: {value_spatial_shapes.dtype}")
-    _check(value_level_start_index.dtype == torch.int32,
-           "value_level_start_index: int32 tensor expected but got a tensor with dtype: "
-           f"{value_level_start_index.dtype}")
+    _check(value_spatial_shapes.dtype in (torch.int32, torch.int64),
+           f"value_spatial_shapes: int32 or int64 tensor expected but got a tensor with dtype: {value_spatial_shapes.dtype}")
+    _check(value_level_start_index.dtype == value_spatial_shapes.dtype,
+           f"value_level_start_index: {value_spatial_shapes.dtype} tensor (as value_spatial_shapes) expected but got a "
+           f"tensor with dtype: {value_level_start_index.dtype}")
     _check(sampling_locations.dtype in _FLOAT_CODES,
            "sampling_locations: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: "
            f"{sampling_locations.dtype}")
@@ -75,8 +81,8 @@ def multi_scale_deformable_attn(value, value_spatial_shapes, value_level_start_i
     with torch.cuda.device(value.device):
         stream = torch.cuda.current_stream().cuda_stream
         rc = lib.mxd_msda_forward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(),
-                                  attn.data_ptr(), output.data_ptr(), _FLOAT_CODES[dt], bs, nk, nh, hd, nl, nl_attn,
-                                  nq, npts, stream)
+                                  attn.data_ptr(), output.data_ptr(), _FLOAT_CODES[dt] | _meta_flag(shapes), bs, nk, nh,
+                                  hd, nl, nl_attn, nq, npts, stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return output
 
@@ -101,7 +107,7 @@ def multi_scale_deformable_attn_backward(value, shape, level_start_index, locati
     grad_value = torch.empty_like(value)
     grad_loc = torch.empty_like(loc)
     grad_attn = torch.empty_like(attn)
-    code = _FLOAT_CODES[dt]
+    code = _FLOAT_CODES[dt] | _meta_flag(shapes)
     ws_bytes = lib.mxd_msda_backward_workspace_bytes(code, bs, nk, nh, hd, nl, nl_attn, nq, npts)
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=value.device)
     with torch.cuda.device(value.device):
@@ -121,8 +127,9 @@ def msda_fused_forward(value, value_spatial_shapes, value_level_start_index, ref
     ``[bs, nq, nh, nl, np, 2]``, attention_logits ``[bs, nq, nh, nl*np]``.  Returns ``[bs, nq, nh*hd]``."""
     _check(value.dtype in _FLOAT_CODES,
            f"value: float16, bfloat16 or float32 tensor expected but got a tensor with dtype: {value.dtype}")
-    _check(value_spatial_shapes.dtype == torch.int32 and value_level_start_index.dtype == torch.int32,
-           "value_spatial_shapes / value_level_start_index: int32 tensors expected")
+    _check(value_spatial_shapes.dtype in (torch.int32, torch.int64) and
+           value_level_start_index.dtype == value_spatial_shapes.dtype,
+           "value_spatial_shapes / value_level_start_index: int32 (or both int64) tensors expected")
     _check(value.dim() == 4, "value: expected [bs, num_keys, num_heads, embed_dims]")
     _check(sampling_offsets.dim() == 6 and sampling_offsets.size(5) == 2,
            "sampling_offsets: expected [bs, num_queries, num_heads, num_levels, num_points, 2]")
@@ -157,7 +164,8 @@ def msda_fused_forward(value, value_spatial_shapes, value_level_start_index, ref
         stream = torch.cuda.current_stream().cuda_stream
         rc = lib.mxd_msda_fused_forward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), ref.data_ptr(),
                                         reference_points.size(3), off.data_ptr(), logits.data_ptr(),
-                                        output.data_ptr(), _FLOAT_CODES[dt], bs, nk, nh, hd, nl, nq, npts, stream)
+                                        output.data_ptr(), _FLOAT_CODES[dt] | _meta_flag(shapes), bs, nk, nh, hd, nl,
+                                        nq, npts, stream)
     _check(rc == 0, _lib.last_error() if rc != 0 else "")
     return output
 
@@ -176,8 +184,9 @@ def msda_fused_backward(value, value_spatial_shapes, value_level_start_index, re
     _, nq, _, nl, npts, _ = sampling_offsets.shape
     _check(tuple(value_spatial_shapes.shape) == (nl, 2) and value_level_start_index.numel() == nl,
            "value_spatial_shapes / value_level_start_index: expected the levels of sampling_offsets")
-    _check(value_spatial_shapes.dtype == torch.int32 and value_level_start_index.dtype == torch.int32,
-           "value_spatial_shapes / value_level_start_index: int32 tensors expected")
+    _check(value_spatial_shapes.dtype in (torch.int32, torch.int64) and
+           value_level_start_index.dtype == value_spatial_shapes.dtype,
+           "value_spatial_shapes / value_level_start_index: int32 (or both int64) tensors expected")
     _check(sampling_offsets.size(0) == bs and sampling_offsets.size(2) == nh,
            "sampling_offsets: batch size / num_heads do not match value")
     _check(reference_points.dim() == 4 and tuple(reference_points.shape[:3]) == (bs, nq, nl),
@@ -195,9 +204,9 @@ def msda_fused_backward(value, value_spatial_shapes, value_level_start_index, re
     _check(all(t.device == value.device for t in tensors), "msda_fused_backward: tensors are on different devices")
     lib = _lib.load()
     dt = value.dtype
-    code = _FLOAT_CODES[dt]
     value = value.contiguous()
     shapes, lsi = value_spatial_shapes.contiguous(), value_level_start_index.contiguous()
+    code = _FLOAT_CODES[dt] | _meta_flag(shapes)
     ref = reference_points.to(dt).contiguous()
     off = sampling_offsets.to(dt).contiguous()
     logits = attention_logits.to(dt).contiguous()

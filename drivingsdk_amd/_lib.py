@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmxd_msda.so")
 
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 BWD_ACCUMULATE = 1
+META_I64 = 0x100  # OR into a dtype code: level metadata tensors hold int64 elements
 
 EXPORTS = (
     "mxd_msda_version",

@@ -33,6 +33,14 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
+// Splits the MXD_META_I64 flag off a dtype argument; returns 1 when it was set.
+static int take_meta_flag(int* dtype)
+{
+    const int f = (*dtype & MXD_META_I64) ? 1 : 0;
+    *dtype &= ~MXD_META_I64;
+    return f;
+}
+
 int elem_size(int dtype)
 {
     switch (dtype) {
@@ -333,6 +341,7 @@ const char* mxd_msda_last_error(void) { return g_err; }
 int mxd_msda_make_plan(int backward, int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn,
                   int64_t nq, int64_t np, int align_bytes, mxd_msda_plan* plan)
 {
+    take_meta_flag(&dtype);
     if (!plan) return fail(MXD_E_NULL, "plan is NULL");
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     int cache = 1;
@@ -358,6 +367,7 @@ static int forward_common(int kind, const void* value, const int32_t* spatial_sh
                           int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np,
                           void* hip_stream, int64_t grid_h = 0, int64_t grid_w = 0)
 {
+    const int meta64 = take_meta_flag(&dtype);
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     const int gka = kind == 1, grid = kind >= 2 ? kind - 1 : 0;
     const char* who = grid ? "mxd_grid_sampler2d_forward" : gka ? "mxd_gka_forward" : "mxd_msda_forward";
@@ -373,6 +383,7 @@ static int forward_common(int kind, const void* value, const int32_t* spatial_sh
     rc = make_plan(0, dtype, d, align, &a.plan, &cache);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.meta_i64 = meta64;
     a.value = value;
     a.shapes = spatial_shapes;
     a.lsi = level_start_index;
@@ -430,6 +441,7 @@ int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, con
                            const void* attn_logits, void* output, int dtype, int64_t bs, int64_t nk, int64_t nh,
                            int64_t hd, int64_t nl, int64_t nq, int64_t np, void* hip_stream)
 {
+    const int meta64 = take_meta_flag(&dtype);
     const Dims d{bs, nk, nh, hd, nl, nl, nq, np};
     int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
@@ -444,6 +456,7 @@ int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, con
     rc = make_plan(0, dtype, d, align, &a.plan);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.meta_i64 = meta64;
     a.value = value;
     a.shapes = spatial_shapes;
     a.lsi = level_start_index;
@@ -460,6 +473,7 @@ int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, con
 size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,
                                          int64_t nl_attn, int64_t nq, int64_t np)
 {
+    take_meta_flag(&dtype);
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     if (check_dims(dtype, d) != MXD_OK) return 0;
     return bwd_layout(dtype, d).total;
@@ -485,6 +499,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
                            int64_t np, int flags, void* hip_stream, int64_t grid_h = 0, int64_t grid_w = 0,
                            const FusedBackward* fused = nullptr)
 {
+    const int meta64 = take_meta_flag(&dtype);
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     const int gka = kind == 1, grid = kind >= 2 ? kind - 1 : 0;
     const char* who = fused  ? "mxd_msda_fused_backward"
@@ -520,6 +535,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     rc = make_plan(1, dtype, d, align, &a.plan);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.meta_i64 = meta64;
     a.value = value;
     a.shapes = spatial_shapes;
     a.lsi = level_start_index;
@@ -578,6 +594,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
 size_t mxd_msda_fused_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd,
                                                int64_t nl, int64_t nq, int64_t np, int ref_dim, int want_grad_ref)
 {
+    take_meta_flag(&dtype);
     const Dims d{bs, nk, nh, hd, nl, nl, nq, np};
     if (check_dims(dtype, d) != MXD_OK || (ref_dim != 2 && ref_dim != 4)) return 0;
     return bwd_layout(dtype, d).total + (want_grad_ref ? fused_part_bytes(d, ref_dim) : 0);
@@ -651,6 +668,7 @@ int mxd_dagg_forward(const void* mc_ms_feat, const int32_t* spatial_shape, const
                      int64_t num_feat, int64_t num_embeds, int64_t num_cams, int64_t num_scale, int64_t num_anchors,
                      int64_t num_pts, int64_t num_groups, void* hip_stream)
 {
+    const int meta64 = take_meta_flag(&dtype);
     Dims d;
     int rc = dagg_dims(dtype, bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups, &d);
     if (rc != MXD_OK) return rc;
@@ -663,6 +681,7 @@ int mxd_dagg_forward(const void* mc_ms_feat, const int32_t* spatial_shape, const
     rc = make_plan(0, dtype, d, align, &a.plan);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.meta_i64 = meta64;
     fill_dagg(&a, num_cams, num_scale);
     a.value = mc_ms_feat;
     a.shapes = spatial_shape;
@@ -678,6 +697,7 @@ int mxd_dagg_forward(const void* mc_ms_feat, const int32_t* spatial_shape, const
 size_t mxd_dagg_backward_workspace_bytes(int dtype, int64_t bs, int64_t num_feat, int64_t num_embeds, int64_t num_cams,
                                          int64_t num_scale, int64_t num_anchors, int64_t num_pts, int64_t num_groups)
 {
+    take_meta_flag(&dtype);
     Dims d;
     if (dagg_dims(dtype, bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups, &d) != MXD_OK)
         return 0;
@@ -691,6 +711,7 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
                       int64_t num_cams, int64_t num_scale, int64_t num_anchors, int64_t num_pts, int64_t num_groups,
                       void* hip_stream)
 {
+    const int meta64 = take_meta_flag(&dtype);
     Dims d;
     int rc = dagg_dims(dtype, bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups, &d);
     if (rc != MXD_OK) return rc;
@@ -717,6 +738,7 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     rc = make_plan(1, dtype, d, align, &a.plan);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.meta_i64 = meta64;
     fill_dagg(&a, num_cams, num_scale);
     a.value = mc_ms_feat;
     a.shapes = spatial_shape;

@@ -21,6 +21,7 @@ struct KArgs {
     const void* value;
     const int32_t* shapes;
     const int32_t* lsi;
+    int32_t meta_i64;      // 1: shapes / lsi are arrays of int64 (MXD_META_I64)
     const void* loc;
     const void* attn;
     void* out;             // forward output
@@ -74,7 +75,9 @@ struct KArgs {
 __device__ inline i32x4 load_level(const KArgs& a, int l)
 {
     if (a.grid) return i32x4{a.grid_h, a.grid_w, 0, 0};
-    return i32x4{a.shapes[2 * l], a.shapes[2 * l + 1], a.lsi[l], 0};
+    // (int64 metadata: the low words of little-endian elements, two int32 apart)
+    const int sh = a.meta_i64;
+    return i32x4{a.shapes[(2 * l) << sh], a.shapes[(2 * l + 1) << sh], a.lsi[l << sh], 0};
 }
 
 // Where a kernel takes the location and the weight of sample s of unit (b, q, h) from.

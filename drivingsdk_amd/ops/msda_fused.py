@@ -45,8 +45,10 @@ class MultiScaleDeformableAttnFusedFunction(Function):
                 attention_logits):
         if torch.numel(value) == 0 or torch.numel(value_spatial_shapes) == 0 or torch.numel(attention_logits) == 0:
             raise Exception("Erorr! Input Tensor can not be a empty Tensor.\n")
-        value_spatial_shapes = value_spatial_shapes.int()
-        value_level_start_index = value_level_start_index.int()
+        # (the reference casts both to int32 here; int64 metadata goes to the library as it is, other types are cast)
+        if value_spatial_shapes.dtype != torch.int64 or value_level_start_index.dtype != torch.int64:
+            value_spatial_shapes = value_spatial_shapes.int()
+            value_level_start_index = value_level_start_index.int()
         reference_points = reference_points.type_as(value)
         sampling_offsets = sampling_offsets.type_as(value)
         attention_logits = attention_logits.type_as(value)

@@ -22,8 +22,10 @@ class MultiScaleDeformableAttnFunction(Function):
                 **kwargs):
         if torch.numel(value) == 0 or torch.numel(value_spatial_shapes) == 0 or torch.numel(attention_weights) == 0:
             raise Exception("Erorr! Input Tensor can not be a empty Tensor.\n")
-        value_spatial_shapes = value_spatial_shapes.int()
-        value_level_start_index = value_level_start_index.int()
+        # (the reference casts both to int32 here; int64 metadata goes to the library as it is, other types are cast)
+        if value_spatial_shapes.dtype != torch.int64 or value_level_start_index.dtype != torch.int64:
+            value_spatial_shapes = value_spatial_shapes.int()
+            value_level_start_index = value_level_start_index.int()
         sampling_locations = sampling_locations.type_as(value)
         attention_weights = attention_weights.type_as(value)
 

@@ -54,6 +54,11 @@ extern "C" {
 #define MXD_DTYPE_F32 0
 #define MXD_DTYPE_F16 1
 #define MXD_DTYPE_BF16 2
+/* OR into `dtype`: spatial_shapes / level_start_index (spatial_shape / scale_start_index) point at int64 elements
+ * instead of int32 ones.  The reference's Python layer receives these tensors as int64 and casts them to int32 on
+ * every call (mx_driving/ops/multi_scale_deformable_attn.py:33-34); with this flag a binding hands them over as they
+ * are and the two cast kernels are not launched.  Values must fit int32 as before. */
+#define MXD_META_I64 0x100
 
 /* error codes */
 #define MXD_OK 0

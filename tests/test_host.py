@@ -127,10 +127,14 @@ def test_binding_dtype_checks_raise_before_any_launch():
     sh, ls = inp.spatial_shapes.int(), inp.level_start_index.int()
     with pytest.raises(RuntimeError, match="value: float16, bfloat16 or float32"):
         _C.multi_scale_deformable_attn(inp.value.double(), sh, ls, inp.sampling_locations, inp.attention_weights)
-    with pytest.raises(RuntimeError, match="value_spatial_shapes: int32"):
+    with pytest.raises(RuntimeError, match="value_spatial_shapes: int32 or int64"):
+        _C.multi_scale_deformable_attn(inp.value, inp.spatial_shapes.float(), ls, inp.sampling_locations,
+                                       inp.attention_weights)
+    # int32 and int64 metadata are both taken, but not one of each
+    with pytest.raises(RuntimeError, match="value_level_start_index: torch.int64 tensor"):
         _C.multi_scale_deformable_attn(inp.value, inp.spatial_shapes, ls, inp.sampling_locations,
                                        inp.attention_weights)
-    with pytest.raises(RuntimeError, match="value_level_start_index: int32"):
+    with pytest.raises(RuntimeError, match="value_level_start_index: torch.int32 tensor"):
         _C.multi_scale_deformable_attn(inp.value, sh, inp.level_start_index, inp.sampling_locations,
                                        inp.attention_weights)
     with pytest.raises(RuntimeError, match="sampling_locations: float16"):

@@ -249,6 +249,32 @@ def test_int64_metadata_and_mixed_float_dtypes_are_coerced(gpu_device):
     assert rel_err(out.double().cpu().numpy(), ref) <= HALF
 
 
+def test_int64_metadata_is_read_in_place(gpu_device):
+    """Level metadata as int64 (what callers hold) is handed to the library with the MXD_META_I64 flag instead of
+    being cast: same results, bit for bit, as with int32 tensors -- forward, backward and the fused form."""
+    from drivingsdk_amd import _C
+    inp = workloads.make_inputs("detr_encoder_bwd", with_grad_output=True, scale_queries=0.03)
+    d = to_device(inp, gpu_device)
+    sh64, ls64 = d.spatial_shapes, d.level_start_index
+    assert sh64.dtype == torch.int64 and ls64.dtype == torch.int64
+    sh32, ls32 = sh64.int(), ls64.int()
+    args = (d.sampling_locations, d.attention_weights)
+    out64 = _C.multi_scale_deformable_attn(d.value, sh64, ls64, *args)
+    out32 = _C.multi_scale_deformable_attn(d.value, sh32, ls32, *args)
+    assert torch.equal(out64, out32)
+    g64 = _C.multi_scale_deformable_attn_backward(d.value, sh64, ls64, *args, d.grad_output)
+    g32 = _C.multi_scale_deformable_attn_backward(d.value, sh32, ls32, *args, d.grad_output)
+    assert torch.equal(g64[1], g32[1]) and torch.equal(g64[2], g32[2])
+    assert rel_err(g64[0].double().cpu().numpy(), g32[0].double().cpu().numpy()) <= 1e-6   # summation order varies
+    bs, nq, nh, nl, npts, _ = d.sampling_locations.shape
+    gen = torch.Generator().manual_seed(8)
+    ref = torch.rand(bs, nq, nl, 2, generator=gen).to(gpu_device)
+    off = torch.randn(bs, nq, nh, nl, npts, 2, generator=gen).to(gpu_device)
+    logits = torch.randn(bs, nq, nh, nl * npts, generator=gen).to(gpu_device)
+    assert torch.equal(_C.msda_fused_forward(d.value, sh64, ls64, ref, off, logits),
+                       _C.msda_fused_forward(d.value, sh32, ls32, ref, off, logits))
+
+
 def test_autocast_runs_in_float32(gpu_device):
     import mx_driving
     inp = workloads.reference_test_inputs([1, 200, 32, 8, 2, 4], seed=5)
