@@ -430,9 +430,9 @@ def main():
                 "kernel_ms": ms}
 
     roof_fwd = roof(bytes_fwd, k["forward_ms"], ["msda_fwd_kernel"])
-    # the backward pass: zero-fill, per-sample dots (grad_attn, grad_loc, keys), grad_value by tile ownership
-    roof_bwd = roof(bytes_bwd, k["backward_with_zero_fill_ms"],
-                    ["msda_fill_zero_kernel", "msda_bwd_kernel", "msda_gradv_tiles_kernel"])
+    # the backward pass: per-sample dots (grad_attn, grad_loc, records; its workgroups also zero-fill the image),
+    # then grad_value by tile ownership
+    roof_bwd = roof(bytes_bwd, k["backward_with_zero_fill_ms"], ["msda_bwd_kernel", "msda_gradv_tiles_kernel"])
     dominant = roof_bwd if roof_bwd["kernel_ms"] >= k["forward_ms"] else roof_fwd
 
     cfg = workloads.WORKLOADS[args.workload]

@@ -41,6 +41,18 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 
     extern __shared__ __align__(16) unsigned char smem[];
     i32x4* lvl = reinterpret_cast<i32x4*>(smem);
+    if constexpr (!SCATTER) {
+        // this workgroup's share of the zero-fill of the image (every workgroup of the launch takes one, also those
+        // without work): the stores ride along with this kernel instead of taking a launch of their own
+        if (a.fill_n4 != 0) {
+            f32x4* img = reinterpret_cast<f32x4*>(a.grad_value);
+            const uint64_t per = (a.fill_n4 + gridDim.x - 1) / gridDim.x;
+            const uint64_t lo = (uint64_t)blockIdx.x * per;
+            const uint64_t hi = lo + per < a.fill_n4 ? lo + per : a.fill_n4;
+            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) img[i] = z;
+        }
+    }
     Work wk;
     if (!decode_block(a.plan, blockIdx.x, a.bs, a.nh, a.nq, &wk)) return;
 

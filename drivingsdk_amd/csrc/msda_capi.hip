@@ -566,7 +566,14 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * nk * nh * hd;
     hipError_t e = hipSuccess;
-    if (!(flags & MXD_BWD_ACCUMULATE)) e = mxd::launch_fill_zero(image, n, stream);
+    // zero-fill of the image: by the first kernel's workgroups when the tile pass is the first to touch it and it
+    // can be written in 16-byte pieces, by a kernel of its own otherwise
+    const bool fill_inside = L.tiles && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 &&
+                             env_int("MXD_MSDA_BWD_FILL_KERNEL", 0) == 0;
+    if (!(flags & MXD_BWD_ACCUMULATE)) {
+        if (fill_inside) a.fill_n4 = n / 4;
+        else e = mxd::launch_fill_zero(image, n, stream);
+    }
     if (e == hipSuccess && part && !a.np_pow2) e = mxd::launch_fill_zero(part, part_bytes / sizeof(float), stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: zero-fill launch failed: %s", who, hipGetErrorString(e));
     const bool atomic_mode = !L.tiles;
@@ -756,7 +763,11 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     a.grad_attn = grad_weights;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * num_feat * num_embeds;
-    hipError_t e = mxd::launch_fill_zero(image, n, stream);
+    hipError_t e = hipSuccess;
+    if (L.tiles && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 && env_int("MXD_MSDA_BWD_FILL_KERNEL", 0) == 0)
+        a.fill_n4 = n / 4;  // zero-filled by the first kernel's workgroups
+    else
+        e = mxd::launch_fill_zero(image, n, stream);
     if (e == hipSuccess && !a.sc_pow2) e = mxd::launch_fill_zero(part, part_bytes / sizeof(float), stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: zero-fill launch failed: %s", hipGetErrorString(e));
     const bool atomic_mode = !L.tiles;

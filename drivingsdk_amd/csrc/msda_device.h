@@ -43,6 +43,8 @@ struct KArgs {
                            // scales across lanes and stored once; otherwise they are added with atomics
     const void* grad_out;  // backward only from here
     float* grad_value;     // fp32 accumulation image of grad_value
+    uint64_t fill_n4;      // first backward kernel, tile mode: 16-byte pieces of the image its workgroups zero-fill
+                           // between them (the image is first touched by the tile pass); 0 = filled by a kernel before
     void* grad_loc;
     void* grad_attn;
     // fused form, backward: `out` holds the forward result (the softmax backward needs, per (query, head), the

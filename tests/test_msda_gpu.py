@@ -433,12 +433,13 @@ def test_backward_accumulate_flag_adds_into_grad_value(gpu_device, name, scale):
 
 @pytest.mark.parametrize("env", [{"MXD_MSDA_BWD_ATOMIC": "1"}, {"MXD_MSDA_BWD_TILE_Q": "64"},
                                  {"MXD_MSDA_BWD_TILE_Q": "256"}, {"MXD_MSDA_TILE_TARGET": "128"},
-                                 {"MXD_MSDA_TILE_TARGET": "1000000"}, {"MXD_MSDA_XCD_MODE": "0"}],
+                                 {"MXD_MSDA_TILE_TARGET": "1000000"}, {"MXD_MSDA_XCD_MODE": "0"},
+                                 {"MXD_MSDA_BWD_FILL_KERNEL": "1"}],
                          ids=lambda e: ",".join(f"{k[9:]}={v}" for k, v in e.items()))
 def test_backward_launch_variants_agree_with_the_oracle(gpu_device, monkeypatch, env):
     """The tuning knobs read at call time select other code paths (one-kernel atomic backward, other
     workgroup sizes of the first kernel, tiles split into very many or no query chunks, plain workgroup
-    mapping); every one of them must give the same gradients."""
+    mapping, zero-fill by a kernel of its own); every one of them must give the same gradients."""
     for k, v in env.items():
         monkeypatch.setenv(k, v)
     for name, scale in (("tiny", 1.0), ("detr_encoder_bwd", 0.25)):
