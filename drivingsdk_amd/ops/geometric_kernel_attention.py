@@ -18,7 +18,8 @@ class GeometricKernelAttentionFunc(Function):
         ctx.value_size = value.size()
         batch_size, num_keys, num_heads, dim = value.size()
         num_queries = attention_weights.size(1)
-        output = value.new_zeros(batch_size, num_queries, num_heads * dim)
+        # (the reference allocates zeros for its kernel to add into; this kernel writes every element)
+        output = value.new_empty(batch_size, num_queries, num_heads * dim)
         _C.geometric_kernel_attention_forward(
             value, spatial_shapes, level_start_index, sampling_locations, attention_weights, output)
         return output
