@@ -36,6 +36,7 @@
 namespace mxd {
 
 constexpr int kLpp = 8;  // lanes per pixel row = pixels per lane group
+constexpr int kWalk = 2; // lists a lane group walks together, one entry of each per trip
 
 // Work item table, evaluated identically by every workgroup.
 struct TileItem {
@@ -332,27 +333,51 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     e = en.w;
                 };
 #pragma unroll
-                for (int i = 0; i < kLpp; i += 4) {
+                for (int i = 0; i < kLpp; i += kWalk) {
                     const int px = grp * kLpp + i;
-                    uint32_t e[4];
+                    uint32_t e[kWalk];
 #pragma unroll
-                    for (int m = 0; m < 4; ++m) e[m] = heads[px + m];
+                    for (int m = 0; m < kWalk; ++m) e[m] = heads[px + m];
                     if (j == 0) {  // same wavefront: ordered after the reads above
 #pragma unroll
-                        for (int m = 0; m < 4; ++m) heads[px + m] = dummy;
+                        for (int m = 0; m < kWalk; ++m) heads[px + m] = dummy;
                     }
-                    while (__ballot((e[0] != dummy) | (e[1] != dummy) | (e[2] != dummy) | (e[3] != dummy))) {
-                        float g[4][CHL], u[4], v[4];
+                    // two sets of rows in flight: the entries and rows of the next trip are requested before the
+                    // rows of this trip are used, so that a long list costs its entries' LDS latency per trip
+                    // and not the latency of a row load (reads past a list's end land on the dummy entry)
+                    float gA[kWalk][CHL], uA[kWalk], vA[kWalk], gB[kWalk][CHL], uB[kWalk], vB[kWalk];
+                    auto use = [&](float (&g)[kWalk][CHL], float (&u)[kWalk], float (&v)[kWalk]) {
 #pragma unroll
-                        for (int m = 0; m < 4; ++m) fetch(e[m], g[m], u[m], v[m]);
-#pragma unroll
-                        for (int m = 0; m < 4; ++m) {
+                        for (int m = 0; m < kWalk; ++m) {
 #pragma unroll
                             for (int c = 0; c < CHL; ++c) {
                                 acc[i + m][c] = __builtin_fmaf(u[m], g[m][c], acc[i + m][c]);
                                 if (i + m + 1 < kLpp)
                                     acc[(i + m + 1) % kLpp][c] = __builtin_fmaf(v[m], g[m][c], acc[(i + m + 1) % kLpp][c]);
                             }
+                        }
+                    };
+                    auto any_left = [&]() {
+                        bool t = false;
+#pragma unroll
+                        for (int m = 0; m < kWalk; ++m) t |= e[m] != dummy;
+                        return __ballot(t) != 0;
+                    };
+                    if (any_left()) {
+#pragma unroll
+                        for (int m = 0; m < kWalk; ++m) fetch(e[m], gA[m], uA[m], vA[m]);
+                        while (true) {
+                            // A holds a trip that has not been used; is there anything after it?
+                            bool pending = any_left();
+#pragma unroll
+                            for (int m = 0; m < kWalk; ++m) fetch(e[m], gB[m], uB[m], vB[m]);
+                            use(gA, uA, vA);
+                            if (!pending) break;  // (B holds dummy entries only)
+                            pending = any_left();
+#pragma unroll
+                            for (int m = 0; m < kWalk; ++m) fetch(e[m], gA[m], uA[m], vA[m]);
+                            use(gB, uB, vB);
+                            if (!pending) break;  // (A holds dummy entries only)
                         }
                     }
                 }
