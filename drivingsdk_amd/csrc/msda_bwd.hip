@@ -214,12 +214,10 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 const T* lg = attn + (((int64_t)wk.b * a.nq + (q < wk.q_end ? q : wk.q_begin)) * a.nh + wk.h) * a.S_full;
                 float m = -__builtin_inff();
                 for (int s = sl; s < a.S; s += kChunk) m = __builtin_fmaxf(m, to_f32(lg[s]));
-#pragma unroll
-                for (int d = 1; d < kChunk; d <<= 1) m = __builtin_fmaxf(m, __shfl_xor(m, d, kWave));
+                m = group_max<4>(m);  // (kChunk = 16 lanes = one DPP row; rows are wholly active or inactive here)
                 float sum = 0.0f;
                 for (int s = sl; s < a.S; s += kChunk) sum += expf(to_f32(lg[s]) - m);
-#pragma unroll
-                for (int d = 1; d < kChunk; d <<= 1) sum += __shfl_xor(sum, d, kWave);
+                sum = group_sum<4>(sum);
                 if (sl == 0) {
                     unit_stats(u)[0] = m;
                     unit_stats(u)[1] = sum;

@@ -433,4 +433,16 @@ __device__ inline float group_sum(float v)
     return v;
 }
 
+// Same for the maximum (lanes of a group that is wholly inactive are not touched).
+template <int LANES_LOG2>
+__device__ inline float group_max(float v)
+{
+    static_assert(LANES_LOG2 <= 4, "within a row of 16 lanes");
+    if constexpr (LANES_LOG2 >= 1) v = __builtin_fmaxf(v, dpp_xchg<0xB1>(v));
+    if constexpr (LANES_LOG2 >= 2) v = __builtin_fmaxf(v, dpp_xchg<0x4E>(v));
+    if constexpr (LANES_LOG2 >= 3) v = __builtin_fmaxf(v, dpp_xchg<0x141>(v));
+    if constexpr (LANES_LOG2 >= 4) v = __builtin_fmaxf(v, dpp_xchg<0x140>(v));
+    return v;
+}
+
 }  // namespace mxd
