@@ -22,7 +22,8 @@
 //   * When the entry storage fills up (or the input ends) the workgroup meets at a barrier and
 //     every lane group walks the lists of its own pixels: one coalesced load of the grad_out
 //     row of the entry's query per group, fma into the registers.  No atomics, no
-//     read-modify-write of shared accumulators.
+//     read-modify-write of shared accumulators.  The walk is pipelined by hand: the entries and
+//     rows of the next trip are requested before the rows of the current trip are used.
 //   * At the end plain 16-byte stores for tiles a single workgroup owns; tiles of hot (coarse)
 //     levels are split over several workgroups by query range and tiles much smaller than the
 //     workgroup are held in several copies: those pass their registers through LDS and add
@@ -314,8 +315,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
             // The lanes of a group read one grad_out row with ONE coalesced load (lane j: channels
             // 4j..4j+3): the memory pipeline's cost is per cache line touched by an instruction.
             // The loop body is branch-free: a list that has ended keeps "reading" the dummy entry.
-            // Four lists are walked together, one entry of each per trip: four independent row
-            // loads in flight, no loop-carried row data (other wavefronts cover the load latency).
+            // kWalk lists are walked together, one entry of each per trip, and two trips are in flight.
             {
                 auto fetch = [&](uint32_t& e, float (&g)[CHL], float& wa, float& wb) {
                     const u32x4 en = ent[e];
