@@ -51,7 +51,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             const uint64_t lo = (uint64_t)blockIdx.x * per;
             const uint64_t hi = lo + per < a.fill_n4 ? lo + per : a.fill_n4;
             const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) img[i] = z;
+            for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) __builtin_nontemporal_store(z, img + i);
         }
     }
     Work wk;
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                                 }
                             }
                         }
-                    } else if constexpr (SRC != kSrcGrid) gattn[sr.w_e] = from_f32<T>(ga);
+                    } else if constexpr (SRC != kSrcGrid) __builtin_nontemporal_store(from_f32<T>(ga), gattn + sr.w_e);
                     if constexpr (FUSED) {
                     } else if constexpr (SRC == kSrcDagg) {
                         // one location serves the scales of its camera and every head: sum over the
@@ -473,8 +473,9 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                             unsafeAtomicAdd(part + 1, gy);
                         }
                     } else if constexpr (SRC != kSrcGka) {  // (pixel-index locations have no gradient)
-                        gloc[2 * sr.loc_e] = from_f32<T>(gx);
-                        gloc[2 * sr.loc_e + 1] = from_f32<T>(gy);
+                        // (streamed out like the records: results should not push value rows out of L2)
+                        __builtin_nontemporal_store(from_f32<T>(gx), gloc + 2 * sr.loc_e);
+                        __builtin_nontemporal_store(from_f32<T>(gy), gloc + 2 * sr.loc_e + 1);
                     }
                     if constexpr (!SCATTER) {
                         // pair records for the tile pass (same decisions as in the counting sweep)

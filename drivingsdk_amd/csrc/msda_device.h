@@ -249,13 +249,14 @@ struct RowIO {
     }
     static __device__ inline void store_global(T* p, const float (&v)[VEC])
     {
+        // (non-temporal: results are not read again by this kernel and should not push value rows out of L2)
         if constexpr (VEC == 1) {
-            *p = from_f32<T>(v[0]);
+            __builtin_nontemporal_store(from_f32<T>(v[0]), p);
         } else {
             vec_t t;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) t[i] = from_f32<T>(v[i]);
-            *reinterpret_cast<vec_t*>(p) = t;
+            __builtin_nontemporal_store(t, reinterpret_cast<vec_t*>(p));
         }
     }
 };
