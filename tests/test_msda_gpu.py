@@ -533,3 +533,31 @@ def test_random_small_problems(gpu_device, seed):
     inp, desc = _random_case(1000 + seed)
     print("case", desc, flush=True)
     _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_small_problems_16bit(gpu_device, seed):
+    """The same kind of problem in float16 (even seeds) and bfloat16 (odd seeds): the float64 oracle runs on the
+    rounded inputs; the results are rounded once more, which for bfloat16 is up to 2^-8 of the largest element."""
+    dtype = torch.float16 if seed % 2 == 0 else torch.bfloat16
+    inp, desc = _random_case(2000 + seed)
+    inp = workloads.MsdaInputs(inp.value.to(dtype), inp.spatial_shapes, inp.level_start_index,
+                               inp.sampling_locations.to(dtype), inp.attention_weights.to(dtype),
+                               inp.grad_output.to(dtype))
+    print("case", desc, dtype, flush=True)
+    tol = HALF if dtype == torch.float16 else 2.0 ** -8
+    ref = oracle_all(inp)
+    got = run_gpu(inp, gpu_device)
+    # 16-bit locations sit on cell edges far more often than float32 ones: the location gradient is compared away
+    # from them only (the oracle and the kernel may take either side of an edge)
+    lo = inp.sampling_locations.double()
+    near = torch.zeros(lo.shape[:-1], dtype=torch.bool)
+    for lvl, (h, w) in enumerate(inp.spatial_shapes.tolist()):
+        w_im, h_im = lo[:, :, :, lvl, :, 0] * w - 0.5, lo[:, :, :, lvl, :, 1] * h - 0.5
+        near[:, :, :, lvl] = ((w_im - w_im.round()).abs() < 2.0 ** -12) | ((h_im - h_im.round()).abs() < 2.0 ** -12)
+    keep = (~near)[..., None].numpy()
+    for name, g_, r_ in zip(("output", "grad_value", "grad_sampling_locations", "grad_attention_weights"), got, ref):
+        r_ = np.asarray(r_)
+        if name == "grad_sampling_locations":
+            g_, r_ = g_ * keep, r_ * keep
+        assert rel_err(g_, r_) <= tol, (name, rel_err(g_, r_), desc)
