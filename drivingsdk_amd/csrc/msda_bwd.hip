@@ -89,23 +89,36 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) cursor[i] = 0;
         __syncthreads();
         const T* loc0 = static_cast<const T*>(a.loc);
-        const int n = (wk.q_end - wk.q_begin) * a.S;
-        for (int i = threadIdx.x; i < n; i += blockDim.x) {
-            const int qr = i / a.S, s = i - qr * a.S;
-            const SampleRef sr = sample_ref<SRC>(a, wk.b, wk.q_begin + qr, wk.h, s);
-            const int l = sr.l;
-            float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
-            if constexpr (FUSED)
-                fused_location(a, static_cast<const T*>(a.ref) + (((int64_t)wk.b * a.nq + wk.q_begin + qr) * a.nl + l) * a.ref_dim,
-                               lvl[l], cx, cy);
-            const bool inside = SRC != kSrcDagg || (cx > 0.0f && cx < 1.0f && cy > 0.0f && cy < 1.0f);
-            const Sample sm = source_geometry<SRC>(cx, cy, lvl[l], a.nk, inside, a.grid);
+        // Records are merged inside aligned groups of 4 samples of a query (merge_pairs_in_quad), here exactly as
+        // where they are written: the samples of a query are padded to a multiple of 4 lanes, and every lane of
+        // the workgroup goes through every trip (the lane exchanges need their partners).
+        const int S4 = (a.S + 3) & ~3;
+        const int n = (wk.q_end - wk.q_begin) * S4;
+        for (int base = 0; base < n; base += blockDim.x) {
+            const int i = base + (int)threadIdx.x;
+            const int qr = i / S4, s = i - qr * S4;
+            const bool act = i < n && s < a.S;
+            int l = 0;
+            Sample sm;
+            sm.cvalid[0] = sm.cvalid[1] = sm.cvalid[2] = sm.cvalid[3] = false;
+            sm.pix[0] = sm.pix[1] = sm.pix[2] = sm.pix[3] = 0;
+            if (act) {
+                const SampleRef sr = sample_ref<SRC>(a, wk.b, wk.q_begin + qr, wk.h, s);
+                l = sr.l;
+                float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
+                if constexpr (FUSED)
+                    fused_location(a, static_cast<const T*>(a.ref) + (((int64_t)wk.b * a.nq + wk.q_begin + qr) * a.nl + l) * a.ref_dim,
+                                   lvl[l], cx, cy);
+                const bool inside = SRC != kSrcDagg || (cx > 0.0f && cx < 1.0f && cy > 0.0f && cy < 1.0f);
+                sm = source_geometry<SRC>(cx, cy, lvl[l], a.nk, inside, a.grid);
+            }
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
-                if ((sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0) {
-                    const int32_t key = sm.cvalid[2 * r] ? sm.pix[2 * r] : sm.pix[2 * r + 1];
+                const bool have = act && (sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0;
+                const int32_t key = sm.cvalid[2 * r] ? sm.pix[2 * r] : sm.pix[2 * r + 1];
+                float za = 0.0f, zb = 0.0f;
+                if (merge_pairs_in_quad(have, key, za, zb))
                     atomicAdd(&cursor[tile_first[l] + ((key - lvl[l].z) >> kTilePxLog2)], 1);
-                }
             }
         }
         __syncthreads();
@@ -236,7 +249,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             // (Only for the plain operator: the other sample sources run with fewer registers and more
             // wavefronts per SIMD without it, which is worth more to them.)
             constexpr int kLaneSamples = 4, kKeep = SRC == kSrcPlain ? 2 : 0, kKeepRegs = kKeep > 0 ? kKeep : 1;
-            float keep_lw[kKeepRegs], keep_lh[kKeepRegs], keep_aw[kKeepRegs], keep_wf[kKeepRegs], keep_hf[kKeepRegs];
+            float keep_lw[kKeepRegs], keep_lh[kKeepRegs], keep_aw[kKeepRegs];
             int32_t keep_pix[kKeepRegs];
             uint32_t keep_fl[kKeepRegs];  // bit 0 valid, bits 1..4 corner valid, bits 8.. level
             constexpr int kUnroll = kKeep > 0 ? kLaneSamples : 1;  // (registers are indexed by ks: unrolled)
@@ -274,8 +287,6 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     keep_lw[ks % kKeepRegs] = sm.lw;
                     keep_lh[ks % kKeepRegs] = sm.lh;
                     keep_aw[ks % kKeepRegs] = aw;
-                    keep_wf[ks % kKeepRegs] = sm.Wf;
-                    keep_hf[ks % kKeepRegs] = sm.Hf;
                     keep_pix[ks % kKeepRegs] = sm.pix[0];
                     keep_fl[ks % kKeepRegs] = (sm.valid ? 1u : 0u) | (sm.cvalid[0] ? 2u : 0u) | (sm.cvalid[1] ? 4u : 0u) |
                                           (sm.cvalid[2] ? 8u : 0u) | (sm.cvalid[3] ? 16u : 0u) | ((uint32_t)l << 8);
@@ -358,6 +369,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 if (i >= entries) break;
                 const int u = i >> 4, sl = i & (kChunk - 1);
                 const int s = c0 + sl, q = q0 + u;
+                // the sample's pair records (upper and lower corners), written after the gradients
+                bool rec_have[2] = {false, false};
+                int32_t rec_key[2] = {0, 0};
+                float rec_wa[2] = {0.f, 0.f}, rec_wb[2] = {0.f, 0.f};
+                int rec_l = 0;
                 if ((q < wk.q_end) && (s < a.S)) {
                     const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
                     int l = sr.l;
@@ -371,8 +387,8 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         sm.valid = (fl & 1u) != 0;
                         sm.lw = keep_lw[ks % kKeepRegs];
                         sm.lh = keep_lh[ks % kKeepRegs];
-                        sm.Wf = keep_wf[ks % kKeepRegs];
-                        sm.Hf = keep_hf[ks % kKeepRegs];
+                        sm.Wf = (float)lvl[l].y;  // (as sample_geometry sets them; only the plain operator keeps samples)
+                        sm.Hf = (float)lvl[l].x;
                         float wt[4];
                         bilinear_weights(sm.lw, sm.lh, wt);
                         const int32_t Wl = lvl[l].y;
@@ -478,19 +494,28 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         __builtin_nontemporal_store(from_f32<T>(gy), gloc + 2 * sr.loc_e + 1);
                     }
                     if constexpr (!SCATTER) {
-                        // pair records for the tile pass (same decisions as in the counting sweep)
+                        rec_l = l;
 #pragma unroll
                         for (int r = 0; r < 2; ++r) {
                             const bool vl = sm.cvalid[2 * r], vr = sm.cvalid[2 * r + 1];
-                            if ((vl || vr) && tile_first[l] >= 0) {
-                                const int32_t key = vl ? sm.pix[2 * r] : sm.pix[2 * r + 1];
-                                const float wa = (vl ? sm.w[2 * r] : sm.w[2 * r + 1]) * aw;
-                                const float wb = (vl && vr) ? sm.w[2 * r + 1] * aw : 0.0f;
-                                const int32_t pos =
-                                    atomicAdd(&cursor[tile_first[l] + ((key - lvl[l].z) >> kTilePxLog2)], 1);
-                                __builtin_nontemporal_store(u32x4{(uint32_t)key, (uint32_t)q, __builtin_bit_cast(uint32_t, wa),
-                                                                  __builtin_bit_cast(uint32_t, wb)}, slab + pos);
-                            }
+                            rec_have[r] = (vl || vr) && tile_first[l] >= 0;
+                            rec_key[r] = vl ? sm.pix[2 * r] : sm.pix[2 * r + 1];
+                            rec_wa[r] = (vl ? sm.w[2 * r] : sm.w[2 * r + 1]) * aw;
+                            rec_wb[r] = (vl && vr) ? sm.w[2 * r + 1] * aw : 0.0f;
+                        }
+                    }
+                }
+                if constexpr (!SCATTER) {
+                    // pair records for the tile pass: the same decisions, lane for lane, as in the counting sweep
+                    // (every lane of an aligned group of 4 takes part in the merge, with or without a record)
+#pragma unroll
+                    for (int r = 0; r < 2; ++r) {
+                        float wa = rec_wa[r], wb = rec_wb[r];
+                        if (merge_pairs_in_quad(rec_have[r], rec_key[r], wa, wb)) {
+                            const int32_t pos =
+                                atomicAdd(&cursor[tile_first[rec_l] + ((rec_key[r] - lvl[rec_l].z) >> kTilePxLog2)], 1);
+                            __builtin_nontemporal_store(u32x4{(uint32_t)rec_key[r], (uint32_t)q, __builtin_bit_cast(uint32_t, wa),
+                                                              __builtin_bit_cast(uint32_t, wb)}, slab + pos);
                         }
                     }
                 }

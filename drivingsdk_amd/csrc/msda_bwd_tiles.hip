@@ -254,7 +254,9 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 uint32_t q = 0;
                 bool spill = false;
                 float wb = 0.f;
-                if (have) {
+                // (a record that does not belong to this tile or names no query of the batch element is dropped:
+                // the run table and the records are only as good as the workspace the caller hands over)
+                if (have && (uint32_t)((int)rc.x - it.p0) < (uint32_t)npx && rc.y < (uint32_t)a.nq) {
                     const uint32_t kx = rc.x, qx = rc.y, ya = rc.z, za = rc.w;
                     q = qx;
                     const int pl = (int)kx - it.p0;

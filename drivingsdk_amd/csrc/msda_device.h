@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "msda_plan.h"
 
 namespace mxd {
@@ -432,6 +434,38 @@ __device__ inline float group_sum(float v)
     if constexpr (LANES_LOG2 >= 5) v += __shfl_xor(v, 16, 64);
     if constexpr (LANES_LOG2 >= 6) v += __shfl_xor(v, 32, 64);
     return v;
+}
+
+// Pair records of one query that start on the same pixel are handed over as one record with the weights added
+// up.  The points of one level of one query sit in neighbouring lanes, and on the coarse levels they often share
+// their cell, so the search is confined to the aligned group of 4 lanes this lane belongs to: the lowest lane
+// that holds a given pixel keeps the record (returns true; wa / wb then carry the sums), the others drop theirs.
+// All four lanes of a group must make the call together; lanes without a record pass have = false.
+// `key` is the record's pixel index (>= 0); the lanes of a group belong to one query.
+__device__ inline bool merge_pairs_in_quad(bool have, int32_t key, float& wa, float& wb)
+{
+    const int j = (int)threadIdx.x & 3;  // lane within the group (workgroups are whole wavefronts)
+    const int32_t k = have ? key : -1;
+    bool keep = have;
+    float sa = wa, sb = wb;
+    // quad_perm [1,2,3,0], [2,3,0,1], [3,0,1,2]: lane j reads lane (j + r) mod 4
+    auto look = [&](auto ctrl, int r) {
+        constexpr int CTRL = decltype(ctrl)::value;
+        const int32_t ko = __builtin_amdgcn_update_dpp(0, k, CTRL, 0xF, 0xF, true);
+        const float ao = dpp_xchg<CTRL>(wa), bo = dpp_xchg<CTRL>(wb);
+        const bool same = have && ko == k;
+        if (same) {
+            if (((j + r) & 3) < j) keep = false;
+            sa += ao;
+            sb += bo;
+        }
+    };
+    look(std::integral_constant<int, 0x39>{}, 1);
+    look(std::integral_constant<int, 0x4E>{}, 2);
+    look(std::integral_constant<int, 0x93>{}, 3);
+    wa = sa;
+    wb = sb;
+    return keep;
 }
 
 // Same for the maximum (lanes of a group that is wholly inactive are not touched).
