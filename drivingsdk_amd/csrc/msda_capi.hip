@@ -169,12 +169,12 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
 int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, mxd::TileArgs* t)
 {
     memset(t, 0, sizeof(*t));
-    // pair records per work item when a hot tile is split: enough items to fill the 512 workgroup
-    // slots of the chip about twice (measured optimum on MI355X; fewer, longer items lose to imbalance,
+    // pair records (counted before merging) per work item when a hot tile is split: enough items to fill the 512
+    // workgroup slots of the chip about twice (measured optimum on MI355X; fewer, longer items lose to imbalance,
     // more, shorter ones to the atomics of their write-out).  Below 8192 records the write-out starts to
     // weigh more and the measured optimum falls more slowly than the problem size: geometric mean of the two
     // (0.17 M samples: 2 100, 0.5 M: 3 600, 1.3 M: 5 700 records per item).
-    int64_t target = 2 * d.bs * d.nh * d.nq * d.nl * d.np / 640;
+    int64_t target = 2 * d.bs * d.nh * d.nq * d.nl * d.np / 512;
     if (target < 8192) target = (int64_t)sqrt(8192.0 * (double)(target > 32 ? target : 32));
     if (target > 32768) target = 32768;
     t->target = env_int("MXD_MSDA_TILE_TARGET", (int)target);
