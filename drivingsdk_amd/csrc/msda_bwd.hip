@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) cursor[i] = 0;
         __syncthreads();
         const T* loc0 = static_cast<const T*>(a.loc);
-        // Records are merged inside aligned groups of 4 samples of a query (merge_pairs_in_quad), here exactly as
+        // Records are merged inside aligned groups of 4 samples of a query (merge_pair_records_in_quad), here exactly as
         // where they are written: the samples of a query are padded to a multiple of 4 lanes, and every lane of
         // the workgroup goes through every trip (the lane exchanges need their partners).
         const int S4 = (a.S + 3) & ~3;
@@ -112,14 +112,18 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 const bool inside = SRC != kSrcDagg || (cx > 0.0f && cx < 1.0f && cy > 0.0f && cy < 1.0f);
                 sm = source_geometry<SRC>(cx, cy, lvl[l], a.nk, inside, a.grid);
             }
+            bool have[2], keep[2];
+            int32_t key[2];
+            float za[2] = {0.f, 0.f}, zb[2] = {0.f, 0.f};
 #pragma unroll
             for (int r = 0; r < 2; ++r) {
-                const bool have = act && (sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0;
-                const int32_t key = sm.cvalid[2 * r] ? sm.pix[2 * r] : sm.pix[2 * r + 1];
-                float za = 0.0f, zb = 0.0f;
-                if (merge_pairs_in_quad(have, key, za, zb))
-                    atomicAdd(&cursor[tile_first[l] + ((key - lvl[l].z) >> kTilePxLog2)], 1);
+                have[r] = act && (sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0;
+                key[r] = sm.cvalid[2 * r] ? sm.pix[2 * r] : sm.pix[2 * r + 1];
             }
+            merge_pair_records_in_quad(have, key, za, zb, keep);
+#pragma unroll
+            for (int r = 0; r < 2; ++r)
+                if (keep[r]) atomicAdd(&cursor[tile_first[l] + ((key[r] - lvl[l].z) >> kTilePxLog2)], 1);
         }
         __syncthreads();
         if (wave == 0) {
@@ -508,14 +512,16 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 if constexpr (!SCATTER) {
                     // pair records for the tile pass: the same decisions, lane for lane, as in the counting sweep
                     // (every lane of an aligned group of 4 takes part in the merge, with or without a record)
+                    bool rec_keep[2];
+                    merge_pair_records_in_quad(rec_have, rec_key, rec_wa, rec_wb, rec_keep);
 #pragma unroll
                     for (int r = 0; r < 2; ++r) {
-                        float wa = rec_wa[r], wb = rec_wb[r];
-                        if (merge_pairs_in_quad(rec_have[r], rec_key[r], wa, wb)) {
+                        if (rec_keep[r]) {
                             const int32_t pos =
                                 atomicAdd(&cursor[tile_first[rec_l] + ((rec_key[r] - lvl[rec_l].z) >> kTilePxLog2)], 1);
-                            __builtin_nontemporal_store(u32x4{(uint32_t)rec_key[r], (uint32_t)q, __builtin_bit_cast(uint32_t, wa),
-                                                              __builtin_bit_cast(uint32_t, wb)}, slab + pos);
+                            __builtin_nontemporal_store(u32x4{(uint32_t)rec_key[r], (uint32_t)q,
+                                                              __builtin_bit_cast(uint32_t, rec_wa[r]),
+                                                              __builtin_bit_cast(uint32_t, rec_wb[r])}, slab + pos);
                         }
                     }
                 }

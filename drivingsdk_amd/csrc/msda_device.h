@@ -438,34 +438,52 @@ __device__ inline float group_sum(float v)
 
 // Pair records of one query that start on the same pixel are handed over as one record with the weights added
 // up.  The points of one level of one query sit in neighbouring lanes, and on the coarse levels they often share
-// their cell, so the search is confined to the aligned group of 4 lanes this lane belongs to: the lowest lane
-// that holds a given pixel keeps the record (returns true; wa / wb then carry the sums), the others drop theirs.
-// All four lanes of a group must make the call together; lanes without a record pass have = false.
-// `key` is the record's pixel index (>= 0); the lanes of a group belong to one query.
-__device__ inline bool merge_pairs_in_quad(bool have, int32_t key, float& wa, float& wb)
+// their cell or sit in cells above one another, so the search is confined to the aligned group of 4 lanes this
+// lane belongs to.  Every lane brings two records -- [0] for the upper corners of its sample, [1] for the lower
+// ones -- and among the records with the same pixel the upper record of the lowest lane that has one keeps it
+// (failing that, the lower record of the lowest lane); keep[] says which of this lane's records survive, and
+// wa / wb of a surviving record carry the sums.  All four lanes of a group must make the call together; a lane
+// without a record passes have = false.  `key` is a record's pixel index (>= 0); the lanes of a group belong to
+// one query.
+__device__ inline void merge_pair_records_in_quad(const bool (&have)[2], const int32_t (&key)[2], float (&wa)[2],
+                                                  float (&wb)[2], bool (&keep)[2])
 {
     const int j = (int)threadIdx.x & 3;  // lane within the group (workgroups are whole wavefronts)
-    const int32_t k = have ? key : -1;
-    bool keep = have;
-    float sa = wa, sb = wb;
+    const int32_t k0 = have[0] ? key[0] : -1, k1 = have[1] ? key[1] : -2;
+    keep[0] = have[0];
+    keep[1] = have[1];
+    float a0 = wa[0], b0 = wb[0], a1 = wa[1], b1 = wb[1];
     // quad_perm [1,2,3,0], [2,3,0,1], [3,0,1,2]: lane j reads lane (j + r) mod 4
     auto look = [&](auto ctrl, int r) {
         constexpr int CTRL = decltype(ctrl)::value;
-        const int32_t ko = __builtin_amdgcn_update_dpp(0, k, CTRL, 0xF, 0xF, true);
-        const float ao = dpp_xchg<CTRL>(wa), bo = dpp_xchg<CTRL>(wb);
-        const bool same = have && ko == k;
-        if (same) {
-            if (((j + r) & 3) < j) keep = false;
-            sa += ao;
-            sb += bo;
+        const int32_t o0 = __builtin_amdgcn_update_dpp(0, k0, CTRL, 0xF, 0xF, true);
+        const int32_t o1 = __builtin_amdgcn_update_dpp(0, k1, CTRL, 0xF, 0xF, true);
+        const float oa0 = dpp_xchg<CTRL>(wa[0]), ob0 = dpp_xchg<CTRL>(wb[0]);
+        const float oa1 = dpp_xchg<CTRL>(wa[1]), ob1 = dpp_xchg<CTRL>(wb[1]);
+        const bool lower = ((j + r) & 3) < j;  // the lane looked at comes before this one
+        if (have[0] && o0 == k0) {
+            if (lower) keep[0] = false;
+            a0 += oa0;
+            b0 += ob0;
+        }
+        if (have[0] && o1 == k0) {  // their lower record joins this upper one
+            a0 += oa1;
+            b0 += ob1;
+        }
+        if (have[1] && o0 == k1) keep[1] = false;  // an upper record takes it
+        if (have[1] && o1 == k1) {
+            if (lower) keep[1] = false;
+            a1 += oa1;
+            b1 += ob1;
         }
     };
     look(std::integral_constant<int, 0x39>{}, 1);
     look(std::integral_constant<int, 0x4E>{}, 2);
     look(std::integral_constant<int, 0x93>{}, 3);
-    wa = sa;
-    wb = sb;
-    return keep;
+    wa[0] = a0;
+    wb[0] = b0;
+    wa[1] = a1;
+    wb[1] = b1;
 }
 
 // Same for the maximum (lanes of a group that is wholly inactive are not touched).
