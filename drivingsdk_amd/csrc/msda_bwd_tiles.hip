@@ -112,6 +112,8 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     static_assert(CHL == 4 && 4 % VEC == 0, "a lane owns one 4-channel piece of a row");
     constexpr int NW = kTilePx / kWave;                 // wavefronts per workgroup
     constexpr uint32_t kDummyOfWave = kTileEntCap - 1;  // last entry slot of every wavefront
+    constexpr int kSlotPxAt = 32 * CH / 4;              // first entry behind wavefront 0's transposition scratch
+    static_assert(kSlotPxAt + kTilePx * 2 / 16 <= (int)kDummyOfWave, "slot map must fit wavefront 0's entry storage");
     __shared__ uint32_t heads[kTilePx];                 // list head per pixel (entry index)
     // entry: {byte offset of the grad_out row, weight for the list's pixel, weight for the
     // next pixel, next entry of the same list}
@@ -123,6 +125,12 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     __shared__ int32_t lv_first[kMaxLevels], lv_nt[kMaxLevels];
     __shared__ int item_ok;
     __shared__ int done_count;
+    // Pixels that collect far more entries than the others (inputs that pile samples on a few pixels) get extra
+    // lists in the slots of the workgroup that no pixel of the tile uses -- when there are such slots.  The first
+    // round counts entries per slot (two 16-bit counters per word); after it the same array holds, per slot,
+    // {first extra slot, number of extra slots (2^k - 1)} as 9 + 4 bits.
+    __shared__ uint32_t slot_info[kTilePx / 2];
+    __shared__ uint32_t spare_next, round1_total;
 
     Work wk;
     if (!decode_block(t.map, blockIdx.x, a.bs, a.nh, t.items_per_bh, &wk)) return;
@@ -136,7 +144,10 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     if (threadIdx.x == 0) {
         item_ok = decode_tile_item(a, t, wk.q_begin, &item_s, lv_first, lv_nt) ? 1 : 0;
         done_count = 0;
+        spare_next = 0;
+        round1_total = 0;
     }
+    if (threadIdx.x < kTilePx / 2) slot_info[threadIdx.x] = 0;
     // an empty list points at the dummy entry of the wavefront that owns the pixel
     heads[threadIdx.x] = (threadIdx.x >> 6) * kTileEntCap + kDummyOfWave;
     __syncthreads();
@@ -154,6 +165,12 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     int copies = 1;
     while (copies < 8 && 2 * copies * npx_pad <= kTilePx) copies *= 2;
     const bool owned = it.exclusive && copies == 1;  // plain stores are enough
+    const int copies_log2 = __builtin_ctz(copies);
+    const int nused = copies * npx_pad;              // slots that stand for a pixel of the tile
+    const int nspare = kTilePx - nused;              // slots free for extra lists
+    const bool can_split = nspare >= kLpp;
+    uint16_t* slot_info16 = reinterpret_cast<uint16_t*>(slot_info);
+    bool first_round = true;                         // (of the first channel pass)
     const uint32_t seg = wave * kTileEntCap;  // this wavefront's entry storage
     uint32_t* run_src = run_src_all + wave * kWave;
     uint32_t* run_pre = run_pre_all + wave * kWave;
@@ -277,6 +294,26 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                         }
                     }
                 }
+                if (can_split && !first_round) {
+                    // entries of a pixel with extra lists are dealt to them by query; a pair entry that moves
+                    // to an extra list leaves its right half to the right pixel's own lists
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) {
+                        if (lst[k] >= 0) {
+                            const uint32_t o = slot_info16[lst[k]];
+                            const uint32_t r = (q >> copies_log2) & (o >> 9);
+                            if (r != 0) {
+                                if (k == 0 && w1[0] != 0.0f) {
+                                    lst[1] = lst[0] + 1;
+                                    w0[1] = w1[0];
+                                    w1[0] = 0.0f;
+                                }
+                                lst[k] = nused + (int)(o & 511u) + (int)r - 1;
+                            }
+                        }
+                    }
+                }
+                const bool count_slots = can_split && first_round;
 #pragma unroll
                 for (int k = 0; k < 2; ++k) {
                     const bool push = lst[k] >= 0;
@@ -289,6 +326,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                             const uint32_t next = atomicExch(&heads[lst[k]], pos);
                             ent[pos] = u32x4{q * row_bytes, __builtin_bit_cast(uint32_t, w0[k]),
                                              __builtin_bit_cast(uint32_t, w1[k]), next};
+                            if (count_slots) atomicAdd(&slot_info[lst[k] >> 1], (lst[k] & 1) ? 0x10000u : 1u);
                         }
                         count += __builtin_popcountll(mask);
                     }
@@ -310,8 +348,27 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 counted = true;
                 if (lane == 0) atomicAdd(&done_count, 1);
             }
+            if (can_split && first_round && lane == 0) atomicAdd(&round1_total, (uint32_t)count);
             __syncthreads();
             const bool all_done = done_count == NW;
+            if (can_split && first_round) {
+                // a slot with more than 1.5 times the average gets extra lists for the rounds to come
+                // (every thread replaces the counter of its own slot; neighbours share a word, not a half)
+                uint32_t o = 0;
+                if (!all_done && tid < nused) {
+                    const uint32_t c = slot_info16[tid];
+                    const float limit = __builtin_fmaxf(1.5f * (float)round1_total / (float)nused, 4.0f);
+                    const uint32_t m = (uint32_t)__builtin_ceilf((float)c / limit);
+                    uint32_t extra = m <= 1 ? 0u : m <= 2 ? 1u : m <= 4 ? 3u : m <= 8 ? 7u : 15u;
+                    if (extra != 0) {
+                        const uint32_t base = atomicAdd(&spare_next, extra);
+                        while (extra != 0 && base + extra > (uint32_t)nspare) extra >>= 1;
+                        if (extra != 0) o = base | (extra << 9);
+                    }
+                }
+                slot_info16[tid] = (uint16_t)o;
+                first_round = false;
+            }
 
             // ---- every group of kLpp lanes walks the lists of its kLpp pixels -----------------
             // The lanes of a group read one grad_out row with ONE coalesced load (lane j: channels
@@ -393,7 +450,21 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         // occupying registers during the rounds)
         int grp_w = grp, lane_w = lane;
         asm volatile("" : "+v"(grp_w), "+v"(lane_w));
-        if (owned && t.store_vec == 4) {
+        // extra lists were handed out: their slots add to their pixels' rows through the atomics below; the map
+        // from extra slot to pixel goes into wavefront 0's entry storage, behind its transposition scratch
+        const bool split = spare_next != 0;  // (uniform; written before the barrier that ended the first round)
+        uint16_t* slot_px = reinterpret_cast<uint16_t*>(&ent[kSlotPxAt]);
+        if (split) {
+            slot_px[tid] = 0xFFFFu;
+            __syncthreads();
+            if (tid < nused) {
+                const uint32_t o = slot_info16[tid];
+                for (uint32_t r = 0; r < (o >> 9); ++r)
+                    if ((o & 511u) + r < (uint32_t)nspare) slot_px[(o & 511u) + r] = (uint16_t)(tid - (tid / npx_pad) * npx_pad);
+            }
+            __syncthreads();
+        }
+        if (owned && !split && t.store_vec == 4) {
             // the lanes of a group hold a whole row of each of their pixels: 16-byte stores
             if (my_ch < hd) {
 #pragma unroll
@@ -442,11 +513,12 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     const int idx = k * kWave + lane_w;
                     const int pl = idx / CH, c = idx % CH;
                     const int vp = px_base + pl;             // pixel slot of the workgroup
-                    const int px = vp - (vp / npx_pad) * npx_pad;  // pixel of the tile (any copy)
-                    if (vp < copies * npx_pad && px < npx && c < nch) {
+                    int px = vp - (vp / npx_pad) * npx_pad;  // pixel of the tile (any copy)
+                    if (vp >= nused) px = split ? (int)slot_px[vp - nused] : npx;  // (0xFFFF: slot without a pixel)
+                    if (px < npx && c < nch) {
                         const float v = __builtin_bit_cast(float, (uint32_t)tr1[idx]);
                         float* dst = gimg + (int64_t)(it.p0 + px) * row_pitch + (int64_t)wk.h * hd + cb + c;
-                        if (!owned || px == 0)
+                        if (!owned || split || px == 0)
                             unsafeAtomicAdd(dst, v);
                         else if (t.accumulate)
                             *dst += v;

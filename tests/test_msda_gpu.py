@@ -511,6 +511,31 @@ def test_documentation_example_all_samples_in_one_pixel(gpu_device, nq):
     assert np.all(np.isfinite(got[2]))
 
 
+@pytest.mark.parametrize("levels,hd", [(((10, 20),), 32), (((23, 31), (9, 7)), 64)], ids=["200px", "713px+63px"])
+def test_hot_pixels_get_extra_lists_in_the_tile_pass(gpu_device, monkeypatch, levels, hd):
+    """A tile smaller than its workgroup leaves lane groups without pixels; pixels that collect far more
+    list entries than the others get extra lists there after the first round (msda_bwd_tiles.hip).  Half of the
+    samples go to three spots of the first level (one of them in its last, partial tile), the others are
+    uniform, and a large work-item size keeps every tile in one work item, so that the rounds after the first
+    run with extra lists, pair entries among the moved ones."""
+    monkeypatch.setenv("MXD_MSDA_TILE_TARGET", "1000000")
+    g = torch.Generator().manual_seed(11)
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh, nl, npts = 2, 6000, 2, len(levels), 4
+    loc = torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.1 - 0.05
+    H, W = levels[0]
+    spots = torch.tensor([[(3.3 + 0.5) / W, (4.6 + 0.5) / H], [(W - 1.4 + 0.5) / W, (H - 1.7 + 0.5) / H],
+                          [(W - 5.25 + 0.5) / W, (H - 1.2 + 0.5) / H]])
+    pick = torch.randint(0, 6, (bs, nq, nh, npts), generator=g)
+    for k in range(3):
+        loc[:, :, :, 0][pick == k] = spots[k]
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g), shapes, lsi, loc,
+                               torch.rand(bs, nq, nh, nl, npts, generator=g), torch.randn(bs, nq, nh * hd, generator=g))
+    errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+    print(levels, errs)
+
+
 def _random_case(seed):
     """A random small problem: odd sizes everywhere, locations reaching outside the image."""
     rng = np.random.default_rng(seed)
