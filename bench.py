@@ -43,6 +43,21 @@ def _event_ms(fn, iters, warmup):
     return start.elapsed_time(stop) / iters
 
 
+def _event_stats_ms(fn, iters):
+    """Median and minimum of single launches: one event pair per call of fn(), recorded back to back on the
+    current stream (an interval runs from the end of the previous call's work to the end of this one's)."""
+    import torch
+
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for start, stop in pairs:
+        start.record()
+        fn()
+        stop.record()
+    torch.cuda.synchronize()
+    ms = sorted(start.elapsed_time(stop) for start, stop in pairs)
+    return {"median": ms[len(ms) // 2], "min": ms[0]}
+
+
 def _kernel_times(d, iters, warmup):
     """Raw C-ABI launches of the three kernels of a step, each timed alone."""
     import torch
@@ -76,6 +91,12 @@ def _kernel_times(d, iters, warmup):
         assert rc == 0, _lib.last_error()
 
     res = {"forward_ms": _event_ms(fwd, iters, warmup), "backward_with_zero_fill_ms": _event_ms(lambda: bwd(0), iters, warmup)}
+    n_single = min(max(iters, 20), 100)
+    res["forward_single_launch_ms"] = _event_stats_ms(fwd, n_single)
+    res["backward_single_launch_ms"] = _event_stats_ms(lambda: bwd(0), n_single)
+    # rate at which the forward moves corner rows (4 per sample) from cache to the CUs
+    samples = bs * nq * nh * nl * npts
+    res["forward_gather_TBps"] = samples * 4 * hd * d.value.element_size() / (res["forward_ms"] * 1e-3) / 1e12
     # gradient accumulation into an existing image (no zero-fill, owned tiles add instead of store)
     res["backward_accumulate_ms"] = _event_ms(lambda: bwd(_lib.BWD_ACCUMULATE), iters, warmup) if code == 0 else None
     return res

@@ -28,6 +28,9 @@
 //     levels are split over several workgroups by query range and tiles much smaller than the
 //     workgroup are held in several copies: those pass their registers through LDS and add
 //     whole rows with a few atomics per workgroup.
+//   * Slots of the workgroup that stand for no pixel take extra lists of pixels that collect
+//     far more entries than the others (decided from the counts of a work item's first round),
+//     so that a hot pixel's entries are walked by several lane groups side by side.
 //
 // Which (level, tile, query chunk) a workgroup works on is derived on the device from
 // spatial_shapes / level_start_index, which never leave device memory; the host only needs
