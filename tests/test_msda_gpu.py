@@ -365,6 +365,40 @@ def test_linearity_at_full_size(gpu_device):
     assert rel_err(lhs.double().cpu().numpy(), rhs.double().cpu().numpy()) <= FWD_FP32
 
 
+@pytest.mark.parametrize("name", ["bevformer_sca", "detr_encoder_bwd"])
+def test_adjoint_identities_at_full_size(gpu_device, name):
+    """Size-independent properties of the backward at the largest shapes: the forward is linear in value and in
+    the attention weights, so <out, g> = <value, grad_value> = <attention_weights, grad_attention_weights> for any
+    g; and along its own direction the location gradient matches a central difference of the forward (bilinear
+    interpolation is piecewise linear in the location, so the difference quotient is exact except for the few
+    samples whose cell the step crosses).  Sums in float64 on the device."""
+    import mx_driving
+    d = to_device(workloads.make_inputs(name, with_grad_output=True), gpu_device)
+    value = d.value.clone().requires_grad_()
+    loc = d.sampling_locations.clone().requires_grad_()
+    attn = d.attention_weights.clone().requires_grad_()
+    out = mx_driving.multi_scale_deformable_attn(value, d.spatial_shapes, d.level_start_index, loc, attn)
+    g = d.grad_output
+    out.backward(g)
+    dot = lambda a, b: float((a.double() * b.double()).sum())
+    lhs = dot(out.detach(), g)
+    scale = float(out.detach().double().norm() * g.double().norm())
+    assert abs(lhs - dot(value.detach(), value.grad)) <= 1e-6 * scale
+    assert abs(lhs - dot(attn.detach(), attn.grad)) <= 1e-6 * scale
+    # directional derivative with respect to the locations, along the gradient itself (a random direction would be
+    # nearly orthogonal to it): steps of at most 1/64 pixel of the finest level
+    direction = loc.grad / loc.grad.abs().max()
+    eps = 1.0 / (64.0 * float(d.spatial_shapes.max()))
+    f = lambda l: mx_driving.multi_scale_deformable_attn(d.value, d.spatial_shapes, d.level_start_index, l,
+                                                         d.attention_weights)
+    with torch.no_grad():
+        fd = dot(f(d.sampling_locations + eps * direction) - f(d.sampling_locations - eps * direction), g) / (2 * eps)
+    an = dot(loc.grad, direction)
+    print(name, "directional derivative: central difference", fd, "gradient", an)
+    # (the few samples that change cell inside the step, and float32 rounding of the locations, leave a per cent)
+    assert abs(fd - an) <= 0.02 * abs(an), (fd, an)
+
+
 def test_c_abi_direct_call_and_error_codes(gpu_device):
     """Straight through the C ABI with raw pointers (what a non-Python host would do)."""
     lib = _lib.load()
