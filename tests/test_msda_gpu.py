@@ -570,6 +570,39 @@ def test_hot_pixels_get_extra_lists_in_the_tile_pass(gpu_device, monkeypatch, le
     print(levels, errs)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_hot_spots_many_rounds(gpu_device, monkeypatch, seed):
+    """Random level shapes whose tiles are partly empty, enough samples for several rounds of the tile pass per
+    work item, a random share of them on a few random spots (anywhere, also across tile and image borders), odd
+    head sizes, float32 and float16; with the default work-item size for even seeds and unsplit tiles for odd ones."""
+    rng = np.random.default_rng(100 + seed)
+    if seed % 2:
+        monkeypatch.setenv("MXD_MSDA_TILE_TARGET", "1000000")
+    nl = int(rng.integers(1, 4))
+    levels = [(int(rng.integers(3, 40)), int(rng.integers(3, 40))) for _ in range(nl)]
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh = int(rng.integers(1, 3)), int(rng.integers(2500, 7000)), int(rng.integers(1, 4))
+    hd = int(rng.choice([8, 20, 32, 48, 64]))
+    npts = int(rng.integers(2, 7))
+    dtype = torch.float16 if seed in (2, 5) else torch.float32
+    g = torch.Generator().manual_seed(200 + seed)
+    loc = torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.2 - 0.1
+    nspots = int(rng.integers(1, 6))
+    spots = torch.rand(nspots, 2, generator=g) * 1.04 - 0.02
+    pick = torch.randint(0, int(nspots / float(rng.uniform(0.2, 0.8))) + 1, loc.shape[:-1], generator=g)
+    for k in range(nspots):
+        loc[pick == k] = spots[k]
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g), shapes, lsi, loc,
+                               torch.rand(bs, nq, nh, nl, npts, generator=g), torch.randn(bs, nq, nh * hd, generator=g))
+    if dtype == torch.float16:
+        inp = workloads.MsdaInputs(*[t.half() if t.is_floating_point() else t for t in inp])
+        errs = _check_all(inp, gpu_device, HALF, HALF)
+    else:
+        errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+    print(seed, levels, (bs, nq, nh, hd, npts), dtype, errs)
+
+
 def _random_case(seed):
     """A random small problem: odd sizes everywhere, locations reaching outside the image."""
     rng = np.random.default_rng(seed)
