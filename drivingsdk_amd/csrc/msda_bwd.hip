@@ -65,12 +65,117 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
 
+    const int LPR = a.plan.lanes_per_row;
+    const int lpr_log2 = __builtin_ctz(LPR);
+    const int U = a.plan.units_per_wave;
+    const int g = lane >> lpr_log2;
+    const int c = lane & (LPR - 1);
+    // lanes per row in the scatter phase: the power of two covering head_dim, within [LPR, 64]
+    int span_log2 = lpr_log2;
+    while ((1 << span_log2) < a.hd && span_log2 < 6) ++span_log2;
+
+    // per-wavefront LDS strip: staged samples, then their four reduced dots
+    unsigned char* strip = smem + kMaxLevels * sizeof(i32x4) +
+                           (size_t)wave * U * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4));
+    Entry* stage = reinterpret_cast<Entry*>(strip);
+    f32x4* dots = reinterpret_cast<f32x4*>(strip + (size_t)U * kChunkStride * sizeof(Entry));
+
+    const T* loc = static_cast<const T*>(a.loc);
+    const T* attn = static_cast<const T*>(a.attn);
+    const T* gout = static_cast<const T*>(a.grad_out);
+    T* gloc = static_cast<T*>(a.grad_loc);
+    T* gattn = static_cast<T*>(a.grad_attn);
+    const T* ref = static_cast<const T*>(a.ref);
+    // fused form: per unit {max logit, sum of exponentials, <forward row, grad_out row>} in the pad entry that
+    // ends the unit's staging strip
+    auto unit_stats = [&](int u) { return reinterpret_cast<float*>(stage + u * kChunkStride + kChunk); };
+
+    const __amdgpu_buffer_rsrc_t vres =
+        make_rsrc(static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes, a.batch_bytes);
+    const __amdgpu_buffer_rsrc_t gres =
+        make_rsrc(reinterpret_cast<const char*>(a.grad_value) + (size_t)wk.b * a.gbatch_bytes, a.gbatch_bytes);
+    const uint32_t head_off = (uint32_t)wk.h * a.hd * sizeof(T);
+    const uint32_t ghead_off = (uint32_t)wk.h * a.hd * 4u;
+
     // ---- records per tile of this workgroup: count, prefix, publish -----------------------
     int32_t* tile_first = reinterpret_cast<int32_t*>(
         smem + kMaxLevels * sizeof(i32x4) +
         (size_t)a.plan.waves_per_block * a.plan.units_per_wave * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4)));
     int32_t* cursor = tile_first + kMaxLevels;  // [tbl_stride] counts, then next free position per tile
     u32x4* slab = nullptr;
+    // ---- geometry of one chunk (kChunk samples of each of the wavefront's units) ----------------
+    // A lane stages entries/64 <= kLaneSamples samples per pass and meets the same samples again when
+    // their dots are reduced: for the first kKeep of them (all, with up to 8 units per wavefront)
+    // fractions, weight, first pixel and validity bits stay in registers until then instead of being
+    // derived from the location a second time.
+    // (Only for the plain operator: the other sample sources run with fewer registers and more
+    // wavefronts per SIMD without it, which is worth more to them.)
+    constexpr int kLaneSamples = 4, kKeep = SRC == kSrcPlain ? 2 : 0, kKeepRegs = kKeep > 0 ? kKeep : 1;
+    constexpr int kUnroll = kKeep > 0 ? kLaneSamples : 1;  // (registers are indexed by ks: unrolled)
+    float keep_lw[kKeepRegs], keep_lh[kKeepRegs], keep_aw[kKeepRegs];
+    int32_t keep_pix[kKeepRegs];
+    uint32_t keep_fl[kKeepRegs];  // bit 0 valid, bits 1..4 corner valid, bits 8.. level
+    // The plain operator stages the first chunk of the first iteration while the records are counted (its
+    // samples' geometry is then derived once, not once for the count and once for the gather).
+    constexpr bool kEarly = SRC == kSrcPlain && !SCATTER;
+    const int entries = U * kChunk;
+    auto geometry = [&](int q0, int c0, auto counting) {
+        constexpr bool COUNT = decltype(counting)::value;
+#pragma unroll kUnroll
+        for (int ks = 0; ks < kLaneSamples; ++ks) {
+            const int i = lane + ks * kWave;
+            if (i >= entries) break;
+            const int u = i >> 4, sl = i & (kChunk - 1);
+            const int s = c0 + sl, q = q0 + u;
+            const bool active = (q < wk.q_end) && (s < a.S);
+            float x = 0.f, y = 0.f, aw = 0.f;
+            int l = 0;
+            if (active) {
+                const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
+                x = to_f32(loc[2 * sr.loc_e]);
+                y = to_f32(loc[2 * sr.loc_e + 1]);
+                if constexpr (SRC == kSrcGrid) aw = 1.0f;  // no weights tensor
+                else aw = to_f32(attn[sr.w_e]);
+                l = sr.l;
+                if constexpr (FUSED) {
+                    fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim, lvl[l], x, y);
+                    aw = expf(aw - unit_stats(u)[0]) / unit_stats(u)[1];
+                }
+            }
+            const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
+            const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside, a.grid);
+            Entry en;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
+                en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
+            }
+            stage[u * kChunkStride + sl] = en;
+            if (ks < kKeep) {
+                keep_lw[ks % kKeepRegs] = sm.lw;
+                keep_lh[ks % kKeepRegs] = sm.lh;
+                keep_aw[ks % kKeepRegs] = aw;
+                keep_pix[ks % kKeepRegs] = sm.pix[0];
+                keep_fl[ks % kKeepRegs] = (sm.valid ? 1u : 0u) | (sm.cvalid[0] ? 2u : 0u) | (sm.cvalid[1] ? 4u : 0u) |
+                                      (sm.cvalid[2] ? 8u : 0u) | (sm.cvalid[3] ? 16u : 0u) | ((uint32_t)l << 8);
+            }
+            if constexpr (COUNT) {
+                // the records these samples will leave, merged exactly as where they are written
+                bool have[2], keep[2];
+                int32_t key[2];
+                float za[2] = {0.f, 0.f}, zb[2] = {0.f, 0.f};
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    have[r] = active && (sm.cvalid[2 * r] || sm.cvalid[2 * r + 1]) && tile_first[l] >= 0;
+                    key[r] = sm.cvalid[2 * r] ? sm.pix[2 * r] : sm.pix[2 * r + 1];
+                }
+                merge_pair_records_in_quad(have, key, za, zb, keep);
+#pragma unroll
+                for (int r = 0; r < 2; ++r)
+                    if (keep[r]) atomicAdd(&cursor[tile_first[l] + ((key[r] - lvl[l].z) >> kTilePxLog2)], 1);
+            }
+        }
+    };
     if constexpr (!SCATTER) {
         const int64_t wg_row = ((int64_t)wk.b * a.nh + wk.h) * a.nwg + wk.q_begin / a.plan.tile_q;
         slab = a.rec + wg_row * a.rec_cap;
@@ -89,15 +194,21 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) cursor[i] = 0;
         __syncthreads();
         const T* loc0 = static_cast<const T*>(a.loc);
+        const int early_units = kEarly ? a.plan.waves_per_block * U : 0;  // their first kChunk samples are counted here:
+        if constexpr (kEarly) {
+            const int q0 = wk.q_begin + wave * U;
+            if (q0 < wk.q_end) geometry(q0, 0, std::true_type{});
+        }
         // Records are merged inside aligned groups of 4 samples of a query (merge_pair_records_in_quad), here exactly as
         // where they are written: the samples of a query are padded to a multiple of 4 lanes, and every lane of
         // the workgroup goes through every trip (the lane exchanges need their partners).
         const int S4 = (a.S + 3) & ~3;
         const int n = (wk.q_end - wk.q_begin) * S4;
-        for (int base = 0; base < n; base += blockDim.x) {
+        const bool all_early = early_units >= wk.q_end - wk.q_begin && a.S <= kChunk;  // nothing left to count
+        for (int base = 0; base < n && !all_early; base += blockDim.x) {
             const int i = base + (int)threadIdx.x;
             const int qr = i / S4, s = i - qr * S4;
-            const bool act = i < n && s < a.S;
+            const bool act = i < n && s < a.S && !(qr < early_units && s < kChunk);
             int l = 0;
             Sample sm;
             sm.cvalid[0] = sm.cvalid[1] = sm.cvalid[2] = sm.cvalid[3] = false;
@@ -148,38 +259,6 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         __syncthreads();  // the cursors are advanced from here on
     }
 
-    const int LPR = a.plan.lanes_per_row;
-    const int lpr_log2 = __builtin_ctz(LPR);
-    const int U = a.plan.units_per_wave;
-    const int g = lane >> lpr_log2;
-    const int c = lane & (LPR - 1);
-    // lanes per row in the scatter phase: the power of two covering head_dim, within [LPR, 64]
-    int span_log2 = lpr_log2;
-    while ((1 << span_log2) < a.hd && span_log2 < 6) ++span_log2;
-
-    // per-wavefront LDS strip: staged samples, then their four reduced dots
-    unsigned char* strip = smem + kMaxLevels * sizeof(i32x4) +
-                           (size_t)wave * U * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4));
-    Entry* stage = reinterpret_cast<Entry*>(strip);
-    f32x4* dots = reinterpret_cast<f32x4*>(strip + (size_t)U * kChunkStride * sizeof(Entry));
-
-    const T* loc = static_cast<const T*>(a.loc);
-    const T* attn = static_cast<const T*>(a.attn);
-    const T* gout = static_cast<const T*>(a.grad_out);
-    T* gloc = static_cast<T*>(a.grad_loc);
-    T* gattn = static_cast<T*>(a.grad_attn);
-    const T* ref = static_cast<const T*>(a.ref);
-    // fused form: per unit {max logit, sum of exponentials, <forward row, grad_out row>} in the pad entry that
-    // ends the unit's staging strip
-    auto unit_stats = [&](int u) { return reinterpret_cast<float*>(stage + u * kChunkStride + kChunk); };
-
-    const __amdgpu_buffer_rsrc_t vres =
-        make_rsrc(static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes, a.batch_bytes);
-    const __amdgpu_buffer_rsrc_t gres =
-        make_rsrc(reinterpret_cast<const char*>(a.grad_value) + (size_t)wk.b * a.gbatch_bytes, a.gbatch_bytes);
-    const uint32_t head_off = (uint32_t)wk.h * a.hd * sizeof(T);
-    const uint32_t ghead_off = (uint32_t)wk.h * a.hd * 4u;
-
     uint32_t choff[NPASS];
 #pragma unroll
     for (int p = 0; p < NPASS; ++p) {
@@ -187,7 +266,6 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         choff[p] = head_off + (ch < a.hd ? ch * (uint32_t)sizeof(T) : 0u);
     }
 
-    const int entries = U * kChunk;
     for (int it = 0; it < a.plan.iters; ++it) {
         const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
         if (q0 >= wk.q_end) break;
@@ -245,57 +323,8 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         }
 
         for (int c0 = 0; c0 < a.S; c0 += kChunk) {
-            // ---- geometry -----------------------------------------------------------------
-            // A lane stages entries/64 <= kLaneSamples samples per pass and meets the same samples again when
-            // their dots are reduced: for the first kKeep of them (all, with up to 8 units per wavefront)
-            // fractions, weight, first pixel and validity bits stay in registers until then instead of being
-            // derived from the location a second time.
-            // (Only for the plain operator: the other sample sources run with fewer registers and more
-            // wavefronts per SIMD without it, which is worth more to them.)
-            constexpr int kLaneSamples = 4, kKeep = SRC == kSrcPlain ? 2 : 0, kKeepRegs = kKeep > 0 ? kKeep : 1;
-            float keep_lw[kKeepRegs], keep_lh[kKeepRegs], keep_aw[kKeepRegs];
-            int32_t keep_pix[kKeepRegs];
-            uint32_t keep_fl[kKeepRegs];  // bit 0 valid, bits 1..4 corner valid, bits 8.. level
-            constexpr int kUnroll = kKeep > 0 ? kLaneSamples : 1;  // (registers are indexed by ks: unrolled)
-#pragma unroll kUnroll
-            for (int ks = 0; ks < kLaneSamples; ++ks) {
-                const int i = lane + ks * kWave;
-                if (i >= entries) break;
-                const int u = i >> 4, sl = i & (kChunk - 1);
-                const int s = c0 + sl, q = q0 + u;
-                const bool active = (q < wk.q_end) && (s < a.S);
-                float x = 0.f, y = 0.f, aw = 0.f;
-                int l = 0;
-                if (active) {
-                    const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
-                    x = to_f32(loc[2 * sr.loc_e]);
-                    y = to_f32(loc[2 * sr.loc_e + 1]);
-                    if constexpr (SRC == kSrcGrid) aw = 1.0f;  // no weights tensor
-                    else aw = to_f32(attn[sr.w_e]);
-                    l = sr.l;
-                    if constexpr (FUSED) {
-                        fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim, lvl[l], x, y);
-                        aw = expf(aw - unit_stats(u)[0]) / unit_stats(u)[1];
-                    }
-                }
-                const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside, a.grid);
-                Entry en;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
-                    en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
-                }
-                stage[u * kChunkStride + sl] = en;
-                if (ks < kKeep) {
-                    keep_lw[ks % kKeepRegs] = sm.lw;
-                    keep_lh[ks % kKeepRegs] = sm.lh;
-                    keep_aw[ks % kKeepRegs] = aw;
-                    keep_pix[ks % kKeepRegs] = sm.pix[0];
-                    keep_fl[ks % kKeepRegs] = (sm.valid ? 1u : 0u) | (sm.cvalid[0] ? 2u : 0u) | (sm.cvalid[1] ? 4u : 0u) |
-                                          (sm.cvalid[2] ? 8u : 0u) | (sm.cvalid[3] ? 16u : 0u) | ((uint32_t)l << 8);
-                }
-            }
+            // ---- geometry (the first chunk of the first iteration was staged while records were counted) ----
+            if (!(kEarly && it == 0 && c0 == 0)) geometry(q0, c0, std::false_type{});
             wave_lds_sync();
 
             // ---- gather and dots -------------------------------------------------------

@@ -123,10 +123,13 @@ static int64_t bwd_tile_q(int dtype, const Dims& d)
     const int64_t least = d.hd * elem_size(dtype) <= 64 ? 64 : 32;
     const int v = env_int("MXD_MSDA_BWD_TILE_Q", 0);
     if (v == 32 || v == 64 || v == 128 || v == 256) return v < least ? least : v;
-    // about 1024 samples per workgroup (measured: 64 queries of 16 samples and 32 queries of 32 samples are the
-    // optima of the encoder and the BEVFormer shapes; 128 queries cost them 3 and 7 %)
+    // about 512 samples per workgroup for rows of up to 128 bytes, 1024 for longer ones (measured: 32 queries of 16
+    // or of 32 samples are the optima of the encoder and the BEVFormer shapes -- with 16 samples per query all of a
+    // workgroup's samples are then staged while its records are counted --, 64 queries of 16 samples that of 512-byte
+    // rows; 128 queries cost 3 to 7 %)
+    const int64_t samples = d.hd * elem_size(dtype) <= 128 ? 512 : 1024;
     int64_t first = 128;
-    while (first > least && first * d.nl * d.np > 1024) first >>= 1;
+    while (first > least && first * d.nl * d.np > samples) first >>= 1;
     for (int64_t tq = first; tq > least; tq >>= 1)
         if (d.bs * d.nh * ((d.nq + tq - 1) / tq) >= 6 * 256) return tq;
     return least;
