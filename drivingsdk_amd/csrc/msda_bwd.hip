@@ -103,6 +103,61 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         (size_t)a.plan.waves_per_block * a.plan.units_per_wave * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4)));
     int32_t* cursor = tile_first + kMaxLevels;  // [tbl_stride] counts, then next free position per tile
     u32x4* slab = nullptr;
+    const int entries = U * kChunk;
+    // ---- per unit: the grad_out row in the value-load layout and, for the fused form, the softmax terms ----
+    float gv[NPASS][VEC];
+    auto unit_prologue = [&](int q0) {
+        // grad_out row of this lane's unit in the value-load layout (for the dots)
+        const int qg = q0 + g;
+        const bool unit_ok = qg < wk.q_end;
+        const T* grow = gout + (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            const int ch = (c + p * LPR) * VEC;
+            if (unit_ok && ch < a.hd) {
+                RowIO<T, VEC>::load_global(grow + ch, gv[p]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) gv[p][e] = 0.0f;
+            }
+        }
+
+        if constexpr (FUSED) {
+            // softmax backward: grad_logit_s = w_s * (grad_w_s - sum_t w_t * grad_w_t), and the sum over the
+            // unit's samples equals the dot product of the forward row with the grad_out row
+            const T* orow = static_cast<const T*>(a.out) +
+                            (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
+            float dsum = 0.0f;
+#pragma unroll
+            for (int p = 0; p < NPASS; ++p) {
+                const int ch = (c + p * LPR) * VEC;
+                if (unit_ok && ch < a.hd) {
+                    float ov[VEC];
+                    RowIO<T, VEC>::load_global(orow + ch, ov);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) dsum = __builtin_fmaf(ov[e], gv[p][e], dsum);
+                }
+            }
+            for (int d = 1; d < LPR; d <<= 1) dsum += __shfl_xor(dsum, d, kWave);
+            if (c == 0 && g < U) unit_stats(g)[2] = dsum;
+            // softmax statistics: lanes 16u..16u+15 share unit u, each takes every 16th logit
+            for (int i = lane; i < entries; i += kWave) {
+                const int u = i >> 4, sl = i & (kChunk - 1), q = q0 + u;
+                const T* lg = attn + (((int64_t)wk.b * a.nq + (q < wk.q_end ? q : wk.q_begin)) * a.nh + wk.h) * a.S_full;
+                float m = -__builtin_inff();
+                for (int s = sl; s < a.S; s += kChunk) m = __builtin_fmaxf(m, to_f32(lg[s]));
+                m = group_max<4>(m);  // (kChunk = 16 lanes = one DPP row; rows are wholly active or inactive here)
+                float sum = 0.0f;
+                for (int s = sl; s < a.S; s += kChunk) sum += expf(to_f32(lg[s]) - m);
+                sum = group_sum<4>(sum);
+                if (sl == 0) {
+                    unit_stats(u)[0] = m;
+                    unit_stats(u)[1] = sum;
+                }
+            }
+            wave_lds_sync();
+        }
+    };
     // ---- geometry of one chunk (kChunk samples of each of the wavefront's units) ----------------
     // A lane stages entries/64 <= kLaneSamples samples per pass and meets the same samples again when
     // their dots are reduced: for the first kKeep of them (all, with up to 8 units per wavefront)
@@ -115,10 +170,9 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     float keep_lw[kKeepRegs], keep_lh[kKeepRegs], keep_aw[kKeepRegs];
     int32_t keep_pix[kKeepRegs];
     uint32_t keep_fl[kKeepRegs];  // bit 0 valid, bits 1..4 corner valid, bits 8.. level
-    // The plain operator stages the first chunk of the first iteration while the records are counted (its
+    // The plain operator and the fused form stage the first chunk of the first iteration while the records are counted (its
     // samples' geometry is then derived once, not once for the count and once for the gather).
-    constexpr bool kEarly = SRC == kSrcPlain && !SCATTER;
-    const int entries = U * kChunk;
+    constexpr bool kEarly = (SRC == kSrcPlain || SRC == kSrcFused) && !SCATTER;
     auto geometry = [&](int q0, int c0, auto counting) {
         constexpr bool COUNT = decltype(counting)::value;
 #pragma unroll kUnroll
@@ -197,7 +251,10 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         const int early_units = kEarly ? a.plan.waves_per_block * U : 0;  // their first kChunk samples are counted here:
         if constexpr (kEarly) {
             const int q0 = wk.q_begin + wave * U;
-            if (q0 < wk.q_end) geometry(q0, 0, std::true_type{});
+            if (q0 < wk.q_end) {
+                if constexpr (FUSED) unit_prologue(q0);  // (the weights need the softmax terms)
+                geometry(q0, 0, std::true_type{});
+            }
         }
         // Records are merged inside aligned groups of 4 samples of a query (merge_pair_records_in_quad), here exactly as
         // where they are written: the samples of a query are padded to a multiple of 4 lanes, and every lane of
@@ -270,57 +327,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
         if (q0 >= wk.q_end) break;
 
-        // grad_out row of this lane's unit in the value-load layout (for the dots)
-        const int qg = q0 + g;
-        const bool unit_ok = qg < wk.q_end;
-        const T* grow = gout + (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
-        float gv[NPASS][VEC];
-#pragma unroll
-        for (int p = 0; p < NPASS; ++p) {
-            const int ch = (c + p * LPR) * VEC;
-            if (unit_ok && ch < a.hd) {
-                RowIO<T, VEC>::load_global(grow + ch, gv[p]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) gv[p][e] = 0.0f;
-            }
-        }
-
-        if constexpr (FUSED) {
-            // softmax backward: grad_logit_s = w_s * (grad_w_s - sum_t w_t * grad_w_t), and the sum over the
-            // unit's samples equals the dot product of the forward row with the grad_out row
-            const T* orow = static_cast<const T*>(a.out) +
-                            (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
-            float dsum = 0.0f;
-#pragma unroll
-            for (int p = 0; p < NPASS; ++p) {
-                const int ch = (c + p * LPR) * VEC;
-                if (unit_ok && ch < a.hd) {
-                    float ov[VEC];
-                    RowIO<T, VEC>::load_global(orow + ch, ov);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) dsum = __builtin_fmaf(ov[e], gv[p][e], dsum);
-                }
-            }
-            for (int d = 1; d < LPR; d <<= 1) dsum += __shfl_xor(dsum, d, kWave);
-            if (c == 0 && g < U) unit_stats(g)[2] = dsum;
-            // softmax statistics: lanes 16u..16u+15 share unit u, each takes every 16th logit
-            for (int i = lane; i < entries; i += kWave) {
-                const int u = i >> 4, sl = i & (kChunk - 1), q = q0 + u;
-                const T* lg = attn + (((int64_t)wk.b * a.nq + (q < wk.q_end ? q : wk.q_begin)) * a.nh + wk.h) * a.S_full;
-                float m = -__builtin_inff();
-                for (int s = sl; s < a.S; s += kChunk) m = __builtin_fmaxf(m, to_f32(lg[s]));
-                m = group_max<4>(m);  // (kChunk = 16 lanes = one DPP row; rows are wholly active or inactive here)
-                float sum = 0.0f;
-                for (int s = sl; s < a.S; s += kChunk) sum += expf(to_f32(lg[s]) - m);
-                sum = group_sum<4>(sum);
-                if (sl == 0) {
-                    unit_stats(u)[0] = m;
-                    unit_stats(u)[1] = sum;
-                }
-            }
-            wave_lds_sync();
-        }
+        if (!(kEarly && FUSED && it == 0)) unit_prologue(q0);  // (the fused form's first iteration: done before the count)
 
         for (int c0 = 0; c0 < a.S; c0 += kChunk) {
             // ---- geometry (the first chunk of the first iteration was staged while records were counted) ----
