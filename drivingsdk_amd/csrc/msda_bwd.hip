@@ -163,9 +163,9 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     // their dots are reduced: for the first kKeep of them (all, with up to 8 units per wavefront)
     // fractions, weight, first pixel and validity bits stay in registers until then instead of being
     // derived from the location a second time.
-    // (Only for the plain operator: the other sample sources run with fewer registers and more
-    // wavefronts per SIMD without it, which is worth more to them.)
-    constexpr int kLaneSamples = 4, kKeep = SRC == kSrcPlain ? 2 : 0, kKeepRegs = kKeep > 0 ? kKeep : 1;
+    // (Only for the plain operator and deformable aggregation: the other sample sources run with fewer registers
+    // and more wavefronts per SIMD without it, which is worth more to them.)
+    constexpr int kLaneSamples = 4, kKeep = (SRC == kSrcPlain || SRC == kSrcDagg) ? 2 : 0, kKeepRegs = kKeep > 0 ? kKeep : 1;
     constexpr int kUnroll = kKeep > 0 ? kLaneSamples : 1;  // (registers are indexed by ks: unrolled)
     float keep_lw[kKeepRegs], keep_lh[kKeepRegs], keep_aw[kKeepRegs];
     int32_t keep_pix[kKeepRegs];
