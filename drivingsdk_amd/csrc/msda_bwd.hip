@@ -25,8 +25,11 @@
 // counts its records per tile in LDS (one geometry sweep over its sampling locations), turns
 // the counts into run starts inside its own slab of the record array, publishes them as its
 // row of the run table, and then -- where it computes grad_loc anyway -- drops every record
-// at the next free position of its tile's run (one LDS integer atomic per record).  Its workgroups also
-// zero-fill the fp32 image of grad_value between them, which the tile pass is the first to touch.
+// at the next free position of its tile's run (one LDS integer atomic per record).  Records of a query
+// that start on the same pixel are merged before they are counted and before they are written.  For the
+// plain operator and the fused form the counting sweep already stages the first chunk of samples of the
+// workgroup's first iteration for the gather, so those samples' geometry is derived once.  Its workgroups
+// also zero-fill the fp32 image of grad_value between them, which the tile pass is the first to touch.
 #include <type_traits>
 
 #include "msda_device.h"
