@@ -449,33 +449,29 @@ __device__ inline void merge_pair_records_in_quad(const bool (&have)[2], const i
                                                   float (&wb)[2], bool (&keep)[2])
 {
     const int j = (int)threadIdx.x & 3;  // lane within the group (workgroups are whole wavefronts)
-    const int32_t k0 = have[0] ? key[0] : -1, k1 = have[1] ? key[1] : -2;
-    keep[0] = have[0];
-    keep[1] = have[1];
-    float a0 = wa[0], b0 = wb[0], a1 = wa[1], b1 = wb[1];
+    // a record that is not there gets a key no other record of the group has: equal keys then mean two records
+    const int32_t k0 = have[0] ? key[0] : -1 - 2 * j, k1 = have[1] ? key[1] : -2 - 2 * j;
+    bool keep0 = have[0], keep1 = have[1];
+    const float wa0 = wa[0], wb0 = wb[0], wa1 = wa[1], wb1 = wb[1];
+    float a0 = wa0, b0 = wb0, a1 = wa1, b1 = wb1;
     // quad_perm [1,2,3,0], [2,3,0,1], [3,0,1,2]: lane j reads lane (j + r) mod 4
     auto look = [&](auto ctrl, int r) {
         constexpr int CTRL = decltype(ctrl)::value;
         const int32_t o0 = __builtin_amdgcn_update_dpp(0, k0, CTRL, 0xF, 0xF, true);
         const int32_t o1 = __builtin_amdgcn_update_dpp(0, k1, CTRL, 0xF, 0xF, true);
-        const float oa0 = dpp_xchg<CTRL>(wa[0]), ob0 = dpp_xchg<CTRL>(wb[0]);
-        const float oa1 = dpp_xchg<CTRL>(wa[1]), ob1 = dpp_xchg<CTRL>(wb[1]);
+        const float oa0 = dpp_xchg<CTRL>(wa0), ob0 = dpp_xchg<CTRL>(wb0);
+        const float oa1 = dpp_xchg<CTRL>(wa1), ob1 = dpp_xchg<CTRL>(wb1);
         const bool lower = ((j + r) & 3) < j;  // the lane looked at comes before this one
-        if (have[0] && o0 == k0) {
-            if (lower) keep[0] = false;
-            a0 += oa0;
-            b0 += ob0;
-        }
-        if (have[0] && o1 == k0) {  // their lower record joins this upper one
-            a0 += oa1;
-            b0 += ob1;
-        }
-        if (have[1] && o0 == k1) keep[1] = false;  // an upper record takes it
-        if (have[1] && o1 == k1) {
-            if (lower) keep[1] = false;
-            a1 += oa1;
-            b1 += ob1;
-        }
+        const bool m00 = o0 == k0, m10 = o1 == k0, m01 = o0 == k1, m11 = o1 == k1;
+        // (adding 0.0f leaves a sum as it is)
+        a0 += m00 ? oa0 : 0.0f;
+        b0 += m00 ? ob0 : 0.0f;
+        a0 += m10 ? oa1 : 0.0f;  // their lower record joins this upper one
+        b0 += m10 ? ob1 : 0.0f;
+        a1 += m11 ? oa1 : 0.0f;
+        b1 += m11 ? ob1 : 0.0f;
+        keep0 = keep0 && !(lower && m00);
+        keep1 = keep1 && !m01 && !(lower && m11);  // (m01: an upper record takes it)
     };
     look(std::integral_constant<int, 0x39>{}, 1);
     look(std::integral_constant<int, 0x4E>{}, 2);
@@ -484,6 +480,8 @@ __device__ inline void merge_pair_records_in_quad(const bool (&have)[2], const i
     wb[0] = b0;
     wa[1] = a1;
     wb[1] = b1;
+    keep[0] = keep0;
+    keep[1] = keep1;
 }
 
 // Same for the maximum (lanes of a group that is wholly inactive are not touched).
