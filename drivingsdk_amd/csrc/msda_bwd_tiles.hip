@@ -172,7 +172,8 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     const int nused = copies * npx_pad;              // slots that stand for a pixel of the tile
     const int nspare = kTilePx - nused;              // slots free for extra lists
     const bool can_split = nspare >= kLpp;
-    uint16_t* slot_info16 = reinterpret_cast<uint16_t*>(slot_info);
+    typedef uint16_t __attribute__((may_alias)) u16_alias;  // halves of LDS words that are also accessed whole
+    u16_alias* slot_info16 = reinterpret_cast<u16_alias*>(slot_info);
     bool first_round = true;                         // (of the first channel pass)
     const uint32_t seg = wave * kTileEntCap;  // this wavefront's entry storage
     uint32_t* run_src = run_src_all + wave * kWave;
@@ -456,7 +457,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         // extra lists were handed out: their slots add to their pixels' rows through the atomics below; the map
         // from extra slot to pixel goes into wavefront 0's entry storage, behind its transposition scratch
         const bool split = spare_next != 0;  // (uniform; written before the barrier that ended the first round)
-        uint16_t* slot_px = reinterpret_cast<uint16_t*>(&ent[kSlotPxAt]);
+        u16_alias* slot_px = reinterpret_cast<u16_alias*>(&ent[kSlotPxAt]);
         if (split) {
             slot_px[tid] = 0xFFFFu;
             __syncthreads();
