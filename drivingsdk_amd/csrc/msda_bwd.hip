@@ -326,9 +326,32 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         choff[p] = head_off + (ch < a.hd ? ch * (uint32_t)sizeof(T) : 0u);
     }
 
+    // A workgroup that passes through one iteration of one chunk (all of the plain operator's samples staged during
+    // the count) collects its records in LDS and writes its slab in whole lines: once every wavefront has gathered,
+    // the staging strips are free, and 32 records per unit (two per sample) fit the first 512 of a unit's 544 bytes.
+    // Record `pos` of the slab lives in strip pos / (32 U) at record pos % (32 U).
+    const bool rec_in_lds = SRC == kSrcPlain && !SCATTER && a.plan.iters == 1 && a.S <= kChunk;
+    const int u32_log2 = __builtin_ctz(U) + 5;
+    auto rec_lds = [&](int pos) {
+        return reinterpret_cast<u32x4*>(smem + kMaxLevels * sizeof(i32x4) +
+                                        (size_t)(pos >> u32_log2) * U * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4))) +
+               (pos & ((1 << u32_log2) - 1));
+    };
+    auto copy_records_out = [&]() {
+        const int total = cursor[a.tbl_stride - 1];  // (exclusive prefix: the entry after the last tile holds the sum)
+        for (int i = threadIdx.x; i < total; i += blockDim.x) __builtin_nontemporal_store(*rec_lds(i), slab + i);
+    };
+
     for (int it = 0; it < a.plan.iters; ++it) {
         const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
-        if (q0 >= wk.q_end) break;
+        if (q0 >= wk.q_end) {
+            if (rec_in_lds) {  // meets the other wavefronts at their two barriers and helps with the copy
+                __syncthreads();
+                __syncthreads();
+                copy_records_out();
+            }
+            break;
+        }
 
         if (!(kEarly && FUSED && it == 0)) unit_prologue(q0);  // (the fused form's first iteration: done before the count)
 
@@ -374,6 +397,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 default: gather_dots(std::integral_constant<int, 6>{}); break;
             }
             wave_lds_sync();
+            if (rec_in_lds) __syncthreads();  // every wavefront's staged entries have been used: the strips take records
             // ---- scatter: grad_value[row_c] += (w_c*attn) * grad_out row --------------------
             // `span` consecutive lanes own consecutive floats of one row, so every atomic
             // instruction covers 64/span rows with fully contiguous 64-byte pieces: the
@@ -558,14 +582,19 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         if (rec_keep[r]) {
                             const int32_t pos =
                                 atomicAdd(&cursor[tile_first[rec_l] + ((rec_key[r] - lvl[rec_l].z) >> kTilePxLog2)], 1);
-                            __builtin_nontemporal_store(u32x4{(uint32_t)rec_key[r], (uint32_t)q,
-                                                              __builtin_bit_cast(uint32_t, rec_wa[r]),
-                                                              __builtin_bit_cast(uint32_t, rec_wb[r])}, slab + pos);
+                            const u32x4 rec = {(uint32_t)rec_key[r], (uint32_t)q, __builtin_bit_cast(uint32_t, rec_wa[r]),
+                                               __builtin_bit_cast(uint32_t, rec_wb[r])};
+                            if (rec_in_lds) *rec_lds(pos) = rec;
+                            else __builtin_nontemporal_store(rec, slab + pos);
                         }
                     }
                 }
             }
             wave_lds_sync();
+            if (rec_in_lds) {  // every wavefront's records are in the strips: the slab is written in whole lines
+                __syncthreads();
+                copy_records_out();
+            }
         }
 
         // slots of levels that attention_weights carries beyond spatial_shapes: zero gradients
