@@ -326,16 +326,19 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         choff[p] = head_off + (ch < a.hd ? ch * (uint32_t)sizeof(T) : 0u);
     }
 
-    // A workgroup that passes through one iteration of one chunk (all of the plain operator's samples staged during
-    // the count) collects its records in LDS and writes its slab in whole lines: once every wavefront has gathered,
-    // the staging strips are free, and 32 records per unit (two per sample) fit the first 512 of a unit's 544 bytes.
-    // Record `pos` of the slab lives in strip pos / (32 U) at record pos % (32 U).
-    const bool rec_in_lds = SRC == kSrcPlain && !SCATTER && a.plan.iters == 1 && a.S <= kChunk;
-    const int u32_log2 = __builtin_ctz(U) + 5;
+    // A workgroup that passes through one iteration of one chunk (all samples of the plain operator and of the fused
+    // form staged during the count) collects its records in LDS and writes its slab in whole lines: once every
+    // wavefront has gathered, the staged entries are free, and a unit's 32 records (two per sample) fit the 16 entries
+    // before its pad entry (which the fused form still needs).  Record `pos` of the slab lives at record pos % 32 of
+    // unit pos / 32 of the workgroup.
+    const bool rec_in_lds = (SRC == kSrcPlain || SRC == kSrcFused) && !SCATTER && a.plan.iters == 1 && a.S <= kChunk;
+    const int u_log2 = __builtin_ctz(U);
     auto rec_lds = [&](int pos) {
+        const int unit = pos >> 5;  // of the workgroup: wavefront unit >> u_log2, its unit & (U - 1)
         return reinterpret_cast<u32x4*>(smem + kMaxLevels * sizeof(i32x4) +
-                                        (size_t)(pos >> u32_log2) * U * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4))) +
-               (pos & ((1 << u32_log2) - 1));
+                                        (size_t)(unit >> u_log2) * U * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4)) +
+                                        (size_t)(unit & (U - 1)) * (kChunkStride * sizeof(Entry))) +
+               (pos & 31);
     };
     auto copy_records_out = [&]() {
         const int total = cursor[a.tbl_stride - 1];  // (exclusive prefix: the entry after the last tile holds the sum)
