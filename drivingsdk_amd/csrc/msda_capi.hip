@@ -268,7 +268,8 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     if (backward) iters = L.tiles ? (int)(L.tile_q / (p->units_per_wave * p->waves_per_block)) : 1;
     int cache = (level_cache && *level_cache && !backward) ? forward_cache_bytes(vec, es, d, p->units_per_wave) : 0;
     if (cache > 0) {
-        // 8 wavefronts share one copy of the cached rows and work through 256 queries; two such workgroups
+        // 8 wavefronts share one copy of the cached rows and work through 128 queries (MXD_MSDA_FWD_WGQ; 256 and
+        // 64 measure within 2 % of it); two such workgroups
         // must fit a CU (80 KiB each), else fewer wavefronts, else no cache
         int waves = 8;
         while (waves > 2 && mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)waves * p->units_per_wave *
@@ -276,7 +277,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
             waves >>= 1;
         if (waves > 2) {
             p->waves_per_block = waves;
-            iters = 256 / (p->units_per_wave * p->waves_per_block);
+            iters = env_int("MXD_MSDA_FWD_WGQ", 128) / (p->units_per_wave * p->waves_per_block);
             if (iters < 1) iters = 1;
         } else {
             cache = 0;
@@ -424,6 +425,7 @@ static int forward_common(int kind, const void* value, const int32_t* spatial_sh
     a.grid_h = (int32_t)grid_h;
     a.grid_w = (int32_t)grid_w;
     a.lds_cache_bytes = cache;
+    a.fwd_ahead = env_int("MXD_MSDA_FWD_AHEAD", 1);
     const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(e));
     return MXD_OK;

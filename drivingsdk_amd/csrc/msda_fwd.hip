@@ -129,6 +129,61 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
     for (int p = 0; p < NPASS; ++p) lds_choff[p] = choff[p] - head_off;
 
     const int entries = U * kChunk;  // staged samples per pass
+
+    // A sample as it is read from memory, and its way into the staging strip.
+    struct RawSample {
+        float x, y, aw;
+        int l, u;
+        bool active;
+    };
+    auto fetch = [&](int q0, int c0, int i) -> RawSample {
+        RawSample r;
+        r.u = i >> 4;
+        const int sl = i & (kChunk - 1);
+        const int s = c0 + sl, q = q0 + r.u;
+        r.active = (i < entries) && (q < wk.q_end) && (s < a.S);
+        r.x = 0.f, r.y = 0.f, r.aw = 0.f, r.l = 0;
+        if (r.active) {
+            const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
+            r.x = to_f32(loc[2 * sr.loc_e]);
+            r.y = to_f32(loc[2 * sr.loc_e + 1]);
+            if constexpr (SRC == kSrcGrid) r.aw = 1.0f;  // no weights tensor
+            else r.aw = to_f32(attn[sr.w_e]);
+            r.l = sr.l;
+            if constexpr (FUSED) {
+                fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + r.l) * a.ref_dim, lvl[r.l], r.x, r.y);
+                r.aw = expf(r.aw - stats[2 * r.u]) / stats[2 * r.u + 1];
+            }
+        }
+        return r;
+    };
+    auto place = [&](const RawSample& r, int i) {
+        const int sl = i & (kChunk - 1);
+        // deformable aggregation samples only strictly inside the image (0 < x, y < 1)
+        const bool inside = SRC != kSrcDagg || (r.x > 0.0f && r.x < 1.0f && r.y > 0.0f && r.y < 1.0f);
+        const Sample sm = source_geometry<SRC>(r.x, r.y, lvl[r.l], a.nk, r.active && inside, a.grid);
+        Entry en;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
+            en.w[k] = sm.valid ? sm.w[k] * r.aw : 0.0f;
+            if constexpr (LDSC) {
+                // cached level: byte offset of the row in the cache; the row of zeros for a corner
+                // outside the image
+                if (r.l >= c_first) en.off[k] = (uint32_t)(sm.cvalid[k] ? sm.pix[k] - c_base : c_rows) * row_bytes;
+            }
+        }
+        stage[r.u * kChunkStride + sl] = en;
+    };
+    // With one chunk of samples per unit and at most two samples per lane, the samples of an iteration are
+    // requested before the gather of the iteration before it, so their way from memory is covered by that gather.
+    const bool ahead = SRC == kSrcPlain && a.S <= kChunk && entries <= 2 * kWave && a.fwd_ahead != 0;
+    RawSample nxt[2];
+    if (ahead) {
+        const int qf = wk.q_begin + wave * U;
+        nxt[0] = fetch(qf, 0, lane);
+        nxt[1] = fetch(qf, 0, lane + kWave);
+    }
     for (int it = 0; it < a.plan.iters; ++it) {
         const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
         if (q0 >= wk.q_end) break;  // wavefront-uniform; no workgroup barrier follows
@@ -160,42 +215,19 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
 
         for (int c0 = 0; c0 < a.S; c0 += kChunk) {
             // ---- geometry: one sample per lane --------------------------------------------
-            for (int i = lane; i < entries; i += kWave) {
-                const int u = i >> 4, sl = i & (kChunk - 1);
-                const int s = c0 + sl, q = q0 + u;
-                const bool active = (q < wk.q_end) && (s < a.S);
-                float x = 0.f, y = 0.f, aw = 0.f;
-                int l = 0;
-                if (active) {
-                    const SampleRef r = sample_ref<SRC>(a, wk.b, q, wk.h, s);
-                    x = to_f32(loc[2 * r.loc_e]);
-                    y = to_f32(loc[2 * r.loc_e + 1]);
-                    if constexpr (SRC == kSrcGrid) aw = 1.0f;  // no weights tensor
-                    else aw = to_f32(attn[r.w_e]);
-                    l = r.l;
-                    if constexpr (FUSED) {
-                        fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim, lvl[l], x, y);
-                        aw = expf(aw - stats[2 * u]) / stats[2 * u + 1];
-                    }
-                }
-                // deformable aggregation samples only strictly inside the image (0 < x, y < 1)
-                const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
-                const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside, a.grid);
-                Entry en;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
-                    en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
-                    if constexpr (LDSC) {
-                        // cached level: byte offset of the row in the cache; the row of zeros for a corner
-                        // outside the image
-                        if (l >= c_first)
-                            en.off[k] = (uint32_t)(sm.cvalid[k] ? sm.pix[k] - c_base : c_rows) * row_bytes;
-                    }
-                }
-                stage[u * kChunkStride + sl] = en;
+            if (ahead) {
+                if (lane < entries) place(nxt[0], lane);
+                if (lane + kWave < entries) place(nxt[1], lane + kWave);
+            } else {
+                for (int i = lane; i < entries; i += kWave) place(fetch(q0, c0, i), i);
             }
             wave_lds_sync();
+            if (ahead) {
+                // the samples of this wavefront's next units are requested now and used after the gather
+                const int qn = q0 + a.plan.waves_per_block * U;
+                nxt[0] = fetch(qn, 0, lane);
+                nxt[1] = fetch(qn, 0, lane + kWave);
+            }
 
             // ---- gather + weighted sum ----------------------------------------------------
             const int ns = (a.S - c0) < kChunk ? (a.S - c0) : kChunk;
