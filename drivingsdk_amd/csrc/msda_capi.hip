@@ -230,7 +230,7 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
 int forward_cache_bytes(int vec, int es, const Dims& d, int units_per_wave)
 {
     const char* forced = getenv("MXD_MSDA_FWD_LDS");
-    const int v = env_int("MXD_MSDA_FWD_LDS", 32768);
+    const int v = env_int("MXD_MSDA_FWD_LDS", 40960);
     if (!(vec * es == 16 && v >= 1024 && v <= 65536)) return 0;
     if (!(forced && *forced)) {
         if (units_per_wave > 8) return 0;
