@@ -59,36 +59,37 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
     // The gather is bound by the vector-memory pipeline (64 bytes per clock per CU); rows held in LDS are read
     // through the LDS pipeline instead, in parallel with it.  Levels are cached from the last one backwards
     // while level_start_index is ascending and the rows from that level's start to the end of value fit.
-    __shared__ int32_t c_first_s, c_base_s, c_rows_s;
     unsigned char* cache = smem + kMaxLevels * sizeof(i32x4) +
                            (size_t)a.plan.waves_per_block * a.plan.units_per_wave * (kChunkStride * sizeof(Entry) + 2 * sizeof(float));
     const uint32_t row_bytes = (uint32_t)a.hd * sizeof(T);
     int c_first = a.nl, c_base = 0, c_rows = 0;
     if constexpr (LDSC) {
-        if (threadIdx.x == 0) {
-            int first = a.nl, base = 0;
-            const int cap_rows = (int)(a.lds_cache_bytes / row_bytes) - 1;  // one more row of zeros
-            for (int l = a.nl - 1; l >= 0; --l) {
-                const int b0 = lvl[l].z;
-                if (b0 < 0 || b0 >= a.nk || a.nk - b0 > cap_rows || (l < a.nl - 1 && b0 > lvl[l + 1].z)) break;
-                first = l;
-                base = b0;
-            }
-            c_first_s = first;
-            c_base_s = base;
-            c_rows_s = first < a.nl ? a.nk - base : 0;
+        // (every thread takes the same decision from the level table in LDS)
+        const int cap_rows = (int)(a.lds_cache_bytes / row_bytes) - 1;  // one more row of zeros
+        for (int l = a.nl - 1; l >= 0; --l) {
+            const int b0 = lvl[l].z;
+            if (b0 < 0 || b0 >= a.nk || a.nk - b0 > cap_rows || (l < a.nl - 1 && b0 > lvl[l + 1].z)) break;
+            c_first = l;
+            c_base = b0;
         }
-        __syncthreads();
-        c_first = c_first_s;
-        c_base = c_base_s;
-        c_rows = c_rows_s;
-        const int pieces = (int)(row_bytes / 16);
+        c_rows = c_first < a.nl ? a.nk - c_base : 0;
+        const int pieces = (int)(row_bytes / 16), total = c_rows * pieces;
         const char* src = static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes +
                           (size_t)c_base * a.pitch_bytes + (size_t)wk.h * row_bytes;
-        for (int i = threadIdx.x; i < c_rows * pieces; i += blockDim.x) {
-            const int row = i / pieces, piece = i - row * pieces;
-            *reinterpret_cast<u32x4*>(cache + (size_t)row * row_bytes + piece * 16) =
-                *reinterpret_cast<const u32x4*>(src + (size_t)row * a.pitch_bytes + piece * 16);
+        // four pieces per thread and trip, all requested before the first is stored
+        for (int i0 = threadIdx.x; i0 < total; i0 += 4 * (int)blockDim.x) {
+            u32x4 piece[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = i0 + j * (int)blockDim.x;
+                const int row = i / pieces, col = i - row * pieces;
+                if (i < total) piece[j] = *reinterpret_cast<const u32x4*>(src + (size_t)row * a.pitch_bytes + col * 16);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = i0 + j * (int)blockDim.x;
+                if (i < total) *reinterpret_cast<u32x4*>(cache + (size_t)i * 16) = piece[j];
+            }
         }
         for (int i = threadIdx.x; i < pieces; i += blockDim.x)
             *reinterpret_cast<u32x4*>(cache + (size_t)c_rows * row_bytes + i * 16) = u32x4{0u, 0u, 0u, 0u};
