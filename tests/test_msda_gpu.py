@@ -496,6 +496,26 @@ def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
         assert rel_err(got, want) <= tol, (name, lds, dtype)
 
 
+@pytest.mark.parametrize("env", [{"MXD_MSDA_FWD_AHEAD": "0"}, {"MXD_MSDA_FWD_AHEAD": "0", "MXD_MSDA_FWD_LDS": "0"},
+                                 {"MXD_MSDA_FWD_LDS": "0"}, {"MXD_MSDA_FWD_WGQ": "64"}, {"MXD_MSDA_FWD_WGQ": "512"},
+                                 {"MXD_MSDA_FWD_LDS": "0", "MXD_MSDA_FWD_ITERS": "3"}],
+                         ids=lambda e: ",".join(f"{k[9:]}={v}" for k, v in e.items()))
+def test_forward_launch_variants_agree(gpu_device, monkeypatch, env):
+    """The forward requests the samples of a wavefront's next units ahead of the gather of the current ones (with and
+    without the level cache, one or several iterations per wavefront, the last one partly filled); every such
+    launch form must give the same output, bit for bit, as the form without it, and meet the oracle."""
+    for name, scale in (("tiny", 1.0), ("detr_encoder", 0.13)):
+        inp = workloads.make_inputs(name, scale_queries=scale)
+        want = oracle_all(inp, with_grads=False)[0]
+        base = run_gpu(inp, gpu_device, with_grads=False)[0]
+        assert rel_err(base, want) <= FWD_FP32, name
+        with monkeypatch.context() as m:
+            for k, v in env.items():
+                m.setenv(k, v)
+            got = run_gpu(inp, gpu_device, with_grads=False)[0]
+        assert np.array_equal(np.asarray(got), np.asarray(base)), (name, env)
+
+
 def test_beyond_the_reference_limits(gpu_device):
     """The reference refuses num_levels * num_points > 64; here 100 samples per (query, head) -- seven staging
     passes, the last one partly filled -- at the largest head_dim (256), forward and gradients."""
