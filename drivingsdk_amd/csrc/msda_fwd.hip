@@ -37,7 +37,7 @@
 
 namespace mxd {
 
-template <typename T, int VEC, int NPASS, int SRC, bool LDSC>
+template <typename T, int VEC, int NPASS, int SRC, bool LDSC, bool AHEAD = false>
 __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs a)
 {
     constexpr bool FUSED = SRC == kSrcFused;
@@ -176,9 +176,11 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
         }
         stage[r.u * kChunkStride + sl] = en;
     };
-    // With one chunk of samples per unit and at most two samples per lane, the samples of an iteration are
-    // requested before the gather of the iteration before it, so their way from memory is covered by that gather.
-    const bool ahead = SRC == kSrcPlain && a.S <= kChunk && entries <= 2 * kWave && a.fwd_ahead != 0;
+    // AHEAD (one chunk of samples per unit, at most two samples per lane; chosen by the launcher): the samples of an
+    // iteration are requested before the gather of the iteration before it, so their way from memory is covered by
+    // that gather.  A template parameter, so that the other forms keep their registers.
+    static_assert(!AHEAD || SRC == kSrcPlain, "look-ahead is built for the plain operator");
+    constexpr bool ahead = AHEAD;
     RawSample nxt[2];
     if (ahead) {
         const int qf = wk.q_begin + wave * U;
@@ -304,23 +306,38 @@ static hipError_t launch_one(const KArgs& a, hipStream_t stream)
         hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcDagg, false>), grid, block, a.plan.lds_bytes, stream, a);
     else if (a.ref != nullptr)
         hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcFused, false>), grid, block, a.plan.lds_bytes, stream, a);
-    else if (a.lds_cache_bytes > 0) {
-        if constexpr (VEC * sizeof(T) == 16) {
-            // more than the 64 KiB of dynamic LDS a kernel gets by default: opt in once per instantiation
-            static bool raised = false;
-            if (!raised) {
-                const hipError_t e = hipFuncSetAttribute(
-                    reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true>),
-                    hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-                if (e != hipSuccess) return e;
-                raised = true;
+    else if (a.ref != nullptr)
+        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcFused, false>), grid, block, a.plan.lds_bytes, stream, a);
+    else {
+        // look-ahead form: one chunk of samples per unit and at most two samples per lane
+        const bool ahead = a.fwd_ahead != 0 && a.S <= kChunk && a.plan.units_per_wave * kChunk <= 2 * kWave;
+        if (a.lds_cache_bytes > 0) {
+            if constexpr (VEC * sizeof(T) == 16) {
+                // more than the 64 KiB of dynamic LDS a kernel gets by default: opt in once per instantiation
+                static bool raised = false;
+                if (!raised) {
+                    hipError_t e = hipFuncSetAttribute(
+                        reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, false>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+                    if (e == hipSuccess)
+                        e = hipFuncSetAttribute(
+                            reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+                    if (e != hipSuccess) return e;
+                    raised = true;
+                }
+                if (ahead)
+                    hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, true>), grid, block, a.plan.lds_bytes, stream, a);
+                else
+                    hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, false>), grid, block, a.plan.lds_bytes, stream, a);
+            } else {
+                return hipErrorInvalidConfiguration;
             }
-            hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true>), grid, block, a.plan.lds_bytes, stream, a);
-        } else {
-            return hipErrorInvalidConfiguration;
-        }
-    } else
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, false>), grid, block, a.plan.lds_bytes, stream, a);
+        } else if (ahead)
+            hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, false, true>), grid, block, a.plan.lds_bytes, stream, a);
+        else
+            hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, false, false>), grid, block, a.plan.lds_bytes, stream, a);
+    }
     return hipGetLastError();
 }
 
