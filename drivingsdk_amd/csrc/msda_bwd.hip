@@ -178,27 +178,37 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     constexpr bool kEarly = (SRC == kSrcPlain || SRC == kSrcFused) && !SCATTER;
     auto geometry = [&](int q0, int c0, auto counting) {
         constexpr bool COUNT = decltype(counting)::value;
-#pragma unroll kUnroll
-        for (int ks = 0; ks < kLaneSamples; ++ks) {
-            const int i = lane + ks * kWave;
-            if (i >= entries) break;
+        // what a lane reads for sample i of the chunk: location, weight, level
+        struct Read {
+            float x, y, aw;
+            int l;
+            bool active;
+        };
+        auto read_sample = [&](int i) -> Read {
+            Read r{0.f, 0.f, 0.f, 0, false};
             const int u = i >> 4, sl = i & (kChunk - 1);
             const int s = c0 + sl, q = q0 + u;
-            const bool active = (q < wk.q_end) && (s < a.S);
-            float x = 0.f, y = 0.f, aw = 0.f;
-            int l = 0;
-            if (active) {
+            r.active = (i < entries) && (q < wk.q_end) && (s < a.S);
+            if (r.active) {
                 const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
-                x = to_f32(loc[2 * sr.loc_e]);
-                y = to_f32(loc[2 * sr.loc_e + 1]);
-                if constexpr (SRC == kSrcGrid) aw = 1.0f;  // no weights tensor
-                else aw = to_f32(attn[sr.w_e]);
-                l = sr.l;
+                r.x = to_f32(loc[2 * sr.loc_e]);
+                r.y = to_f32(loc[2 * sr.loc_e + 1]);
+                if constexpr (SRC == kSrcGrid) r.aw = 1.0f;  // no weights tensor
+                else r.aw = to_f32(attn[sr.w_e]);
+                r.l = sr.l;
                 if constexpr (FUSED) {
-                    fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + l) * a.ref_dim, lvl[l], x, y);
-                    aw = expf(aw - unit_stats(u)[0]) / unit_stats(u)[1];
+                    fused_location(a, ref + (((int64_t)wk.b * a.nq + q) * a.nl + r.l) * a.ref_dim, lvl[r.l], r.x, r.y);
+                    r.aw = expf(r.aw - unit_stats(u)[0]) / unit_stats(u)[1];
                 }
             }
+            return r;
+        };
+        auto stage_sample = [&](auto ks_c, int i, const Read& rd) {
+            constexpr int ks = decltype(ks_c)::value;  // (which registers keep the sample; i = lane + ks * 64 then)
+            const int u = i >> 4, sl = i & (kChunk - 1);
+            const bool active = rd.active;
+            const float x = rd.x, y = rd.y, aw = rd.aw;
+            const int l = rd.l;
             const bool inside = SRC != kSrcDagg || (x > 0.0f && x < 1.0f && y > 0.0f && y < 1.0f);
             const Sample sm = source_geometry<SRC>(x, y, lvl[l], a.nk, active && inside, a.grid);
             Entry en;
@@ -231,6 +241,23 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 for (int r = 0; r < 2; ++r)
                     if (keep[r]) atomicAdd(&cursor[tile_first[l] + ((key[r] - lvl[l].z) >> kTilePxLog2)], 1);
             }
+        };
+        if constexpr (kUnroll == kLaneSamples) {
+            // two samples are read together (one trip to memory instead of two), then staged
+            static_assert(kLaneSamples == 4, "written out for four samples per lane");
+            {
+                const Read r0 = read_sample(lane), r1 = read_sample(lane + kWave);
+                if (lane < entries) stage_sample(std::integral_constant<int, 0>{}, lane, r0);
+                if (lane + kWave < entries) stage_sample(std::integral_constant<int, 1>{}, lane + kWave, r1);
+            }
+            if (lane + 2 * kWave < entries) {
+                const Read r2 = read_sample(lane + 2 * kWave), r3 = read_sample(lane + 3 * kWave);
+                stage_sample(std::integral_constant<int, 2>{}, lane + 2 * kWave, r2);
+                if (lane + 3 * kWave < entries) stage_sample(std::integral_constant<int, 3>{}, lane + 3 * kWave, r3);
+            }
+        } else {
+            for (int i = lane; i < entries && i < kLaneSamples * kWave; i += kWave)
+                stage_sample(std::integral_constant<int, 0>{}, i, read_sample(i));
         }
     };
     if constexpr (!SCATTER) {
