@@ -17,6 +17,8 @@ META_I64 = 0x100  # OR into a dtype code: level metadata tensors hold int64 elem
 EXPORTS = (
     "mxd_msda_version",
     "mxd_msda_last_error",
+    "mxd_msda_init",
+    "mxd_msda_reload_tuning",
     "mxd_msda_make_plan",
     "mxd_msda_decode_block",
     "mxd_msda_forward",
@@ -68,6 +70,10 @@ def load():
     lib.mxd_msda_version.argtypes = []
     lib.mxd_msda_last_error.restype = ctypes.c_char_p
     lib.mxd_msda_last_error.argtypes = []
+    lib.mxd_msda_init.restype = ci
+    lib.mxd_msda_init.argtypes = []
+    lib.mxd_msda_reload_tuning.restype = None
+    lib.mxd_msda_reload_tuning.argtypes = []
     lib.mxd_msda_make_plan.restype = ci
     lib.mxd_msda_make_plan.argtypes = [ci, ci] + [i64] * 8 + [ci, ctypes.POINTER(Plan)]
     lib.mxd_msda_decode_block.restype = ci
@@ -105,6 +111,11 @@ def load():
     lib.mxd_grid_sampler2d_backward.argtypes = [p] * 6 + [ctypes.c_size_t, ci] + [i64] * 6 + [ci] * 3 + [p]
     _lib = lib
     return lib
+
+
+def reload_tuning():
+    """Have the library read its MXD_MSDA_* environment variables again (they are read once per process)."""
+    load().mxd_msda_reload_tuning()
 
 
 def last_error():

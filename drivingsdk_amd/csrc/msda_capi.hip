@@ -9,10 +9,16 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "msda_device.h"
 
 namespace mxd {
 hipError_t launch_forward(int dtype, const KArgs& a, hipStream_t stream);
+hipError_t launch_forward_cu(int dtype, const KArgs& a, hipStream_t stream);
+hipError_t raise_forward_lds();
+hipError_t raise_forward_cu_lds();
 hipError_t launch_backward(int dtype, const KArgs& a, bool scatter, hipStream_t stream);
 hipError_t launch_gradv_tiles(int dtype, const KArgs& a, const TileArgs& t, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t stream);
@@ -57,6 +63,70 @@ int env_int(const char* name, int dflt)
     return (v && *v) ? atoi(v) : dflt;
 }
 
+// Tuning knobs, read from the environment once per process (mxd_msda_reload_tuning() reads them again: a hook for
+// tests and experiments, not to be called while other threads are inside the library).
+struct Tuning {
+    int xcd_mode;        // MXD_MSDA_XCD_MODE: 0 = plain workgroup mapping, -1 = by head count
+    int bwd_tile_q;      // MXD_MSDA_BWD_TILE_Q: queries per workgroup of the first backward kernel, 0 = chosen here
+    int bwd_atomic;      // MXD_MSDA_BWD_ATOMIC: 1 = one-kernel backward with global atomics
+    int tile_target;     // MXD_MSDA_TILE_TARGET: pair records per work item of the tile pass, 0 = chosen here
+    int fwd_lds;         // MXD_MSDA_FWD_LDS: bytes of the general forward's level cache, -1 = by estimate
+    int fwd_iters;       // MXD_MSDA_FWD_ITERS
+    int fwd_wgq;         // MXD_MSDA_FWD_WGQ: queries per workgroup of the general forward with a level cache
+    int fwd_ahead;       // MXD_MSDA_FWD_AHEAD
+    int fwd_cu;          // MXD_MSDA_FWD_CU: 0 = never use the one-workgroup-per-CU forward, 1 = whenever it can run,
+                         // -1 = for problems large enough to pay for it
+    int fwd_cu_wgs;      // MXD_MSDA_FWD_CU_WGS: its workgroups per (batch, head), 0 = chosen here
+    int bwd_fill_kernel; // MXD_MSDA_BWD_FILL_KERNEL: 1 = zero-fill by a kernel of its own
+};
+Tuning g_tuning;
+std::once_flag g_tuning_once;
+
+void read_tuning()
+{
+    Tuning t;
+    t.xcd_mode = env_int("MXD_MSDA_XCD_MODE", -1);
+    t.bwd_tile_q = env_int("MXD_MSDA_BWD_TILE_Q", 0);
+    t.bwd_atomic = env_int("MXD_MSDA_BWD_ATOMIC", 0);
+    t.tile_target = env_int("MXD_MSDA_TILE_TARGET", 0);
+    t.fwd_lds = env_int("MXD_MSDA_FWD_LDS", -1);
+    t.fwd_iters = env_int("MXD_MSDA_FWD_ITERS", 1);
+    t.fwd_wgq = env_int("MXD_MSDA_FWD_WGQ", 128);
+    t.fwd_ahead = env_int("MXD_MSDA_FWD_AHEAD", 1);
+    t.fwd_cu = env_int("MXD_MSDA_FWD_CU", -1);
+    t.fwd_cu_wgs = env_int("MXD_MSDA_FWD_CU_WGS", 0);
+    t.bwd_fill_kernel = env_int("MXD_MSDA_BWD_FILL_KERNEL", 0);
+    g_tuning = t;
+}
+
+const Tuning& tuning()
+{
+    std::call_once(g_tuning_once, read_tuning);
+    return g_tuning;
+}
+
+// Per-device set-up, done once per device on the first call that needs it (or by mxd_msda_init()): the forward
+// kernels that use more than 64 KiB of dynamic LDS opt in.
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_device_ready[kMaxDevices];
+std::mutex g_device_mutex;
+
+int ensure_device_ready()
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "hipGetDevice failed: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(MXD_E_LAUNCH, "device ordinal %d is beyond what this build keeps state for", dev);
+    if (g_device_ready[dev].load(std::memory_order_acquire)) return MXD_OK;
+    std::lock_guard<std::mutex> lock(g_device_mutex);
+    if (g_device_ready[dev].load(std::memory_order_relaxed)) return MXD_OK;
+    e = mxd::raise_forward_lds();
+    if (e == hipSuccess) e = mxd::raise_forward_cu_lds();
+    if (e != hipSuccess) return fail(MXD_E_LAUNCH, "raising the dynamic LDS limit failed: %s", hipGetErrorString(e));
+    g_device_ready[dev].store(1, std::memory_order_release);
+    return MXD_OK;
+}
+
 struct Dims {
     int64_t bs, nk, nh, hd, nl, nl_attn, nq, np;
 };
@@ -88,7 +158,7 @@ int check_dims(int dtype, const Dims& d)
 int64_t fill_xcd_map(mxd_msda_plan* p, int64_t bs, int64_t nh, int64_t ntiles)
 {
     p->ntiles = (int32_t)ntiles;
-    const int mode_override = env_int("MXD_MSDA_XCD_MODE", -1);
+    const int mode_override = tuning().xcd_mode;
     if (mode_override != 0 && nh % mxd::kNumXcd == 0) {
         p->xcd_mode = 1;
         p->heads_per_xcd = (int32_t)(nh / mxd::kNumXcd);
@@ -110,6 +180,31 @@ int64_t fill_xcd_map(mxd_msda_plan* p, int64_t bs, int64_t nh, int64_t ntiles)
     return bs * nh * ntiles;
 }
 
+// Bytes of dynamic LDS of the first backward kernel for a plan (tile mode: with the per-tile counters).
+size_t backward_lds_bytes(int units_per_wave, int waves, bool tiles, int64_t tbl_stride)
+{
+    const size_t per_unit = mxd::kChunkStride * sizeof(mxd::Entry) + mxd::kChunk * sizeof(mxd::f32x4);
+    size_t n = mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)waves * units_per_wave * per_unit;
+    if (tiles) n += (size_t)(mxd::kMaxLevels + tbl_stride) * sizeof(int32_t);
+    return n;
+}
+
+// Row geometry of a problem: elements per lane, lanes per row, row passes.
+void row_geometry(int es, int64_t hd, int align_bytes, int* vec_out, int* lpr_out, int* npass_out)
+{
+    if (align_bytes < es) align_bytes = es;
+    int vec = 16 / es;
+    while (vec > 1 && (hd % vec != 0 || align_bytes < vec * es)) vec >>= 1;
+    const int lanes_needed = (int)((hd + vec - 1) / vec);
+    int lpr = 4;
+    while (lpr < lanes_needed && lpr < mxd::kWave) lpr <<= 1;
+    int npass = (lanes_needed + lpr - 1) / lpr;
+    if (npass == 3) npass = 4;
+    *vec_out = vec;
+    *lpr_out = lpr;
+    *npass_out = npass;
+}
+
 // How the backward pass is laid out for a problem size: whether grad_value goes through the
 // tile-ownership pass (and then the hand-over buffers between its two kernels) or through
 // global atomics, and where things live in the caller's workspace.
@@ -122,7 +217,7 @@ static int64_t bwd_tile_q(int dtype, const Dims& d)
 {
     // (units with very many samples -- deformable aggregation's 312 -- measured 1 to 2 % better with 64)
     const int64_t least = (d.hd * elem_size(dtype) <= 64 || d.nl * d.np >= 256) ? 64 : 32;
-    const int v = env_int("MXD_MSDA_BWD_TILE_Q", 0);
+    const int v = tuning().bwd_tile_q;
     if (v == 32 || v == 64 || v == 128 || v == 256) return v < least ? least : v;
     // about 512 samples per workgroup for rows of up to 128 bytes, 1024 for longer ones (measured: 32 queries of 16
     // or of 32 samples are the optima of the encoder and the BEVFormer shapes -- with 16 samples per query all of a
@@ -155,8 +250,13 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
     // (the kernels leave out levels that would not fit, which can only happen for overlapping levels)
     L.tbl_stride = d.nk / mxd::kTilePx + d.nl + 1;
     const int64_t tbl = d.bs * d.nh * L.nwg * L.tbl_stride * 4;
-    L.tiles = env_int("MXD_MSDA_BWD_ATOMIC", 0) == 0 &&
-              L.tbl_stride <= 4096 &&                      // counters of the first kernel live in LDS
+    // dynamic LDS of the first kernel with the most units per wavefront the row can have (16-byte aligned pointers)
+    int vec, lpr, npass;
+    row_geometry(elem_size(dtype), d.hd, 16, &vec, &lpr, &npass);
+    const size_t lds = backward_lds_bytes(mxd::kWave / lpr, 4, true, L.tbl_stride);
+    L.tiles = tuning().bwd_atomic == 0 &&
+              L.tbl_stride <= 4096 &&                      // counters of the first kernel live in LDS ...
+              lds <= 64 * 1024 &&                          // ... and its strips and counters fit the default limit
               tbl <= (int64_t(1) << 28) &&                 // run table of at most 256 MiB
               L.nwg * L.rec_cap < (int64_t(1) << 31) &&    // 32-bit record indices within a (batch, head)
               d.nq * d.nh * d.hd * 4 < (int64_t(1) << 31); // grad_output rows addressed with 32-bit byte offsets
@@ -202,7 +302,7 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
         }
         target = (per_tile + best_c - 1) / best_c;
     }
-    t->target = env_int("MXD_MSDA_TILE_TARGET", (int)target);
+    t->target = tuning().tile_target > 0 ? tuning().tile_target : (int)target;
     if (t->target < 128) t->target = 128;
     t->max_chunks = 64;
     // work items per (batch, head): sum over levels of tiles*chunks <= 2*nl*nq*np/target + nl + sum of tiles
@@ -229,10 +329,10 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
 // MXD_MSDA_FWD_LDS set in the environment overrides the estimate (0 = off, bytes = on).
 int forward_cache_bytes(int vec, int es, const Dims& d, int units_per_wave)
 {
-    const char* forced = getenv("MXD_MSDA_FWD_LDS");
-    const int v = env_int("MXD_MSDA_FWD_LDS", 40960);
+    const bool forced = tuning().fwd_lds >= 0;
+    const int v = forced ? tuning().fwd_lds : 40960;
     if (!(vec * es == 16 && v >= 1024 && v <= 65536)) return 0;
-    if (!(forced && *forced)) {
+    if (!forced) {
         if (units_per_wave > 8) return 0;
         double last = (double)d.nk;
         if (d.nl > 1) last = (double)d.nk * 3.0 / ((double)(int64_t(1) << (2 * (d.nl < 16 ? d.nl : 16))) - 1.0);
@@ -241,27 +341,103 @@ int forward_cache_bytes(int vec, int es, const Dims& d, int units_per_wave)
     return v & ~15;
 }
 
+// Rows of the last levels that an LDS cache of `cap_rows` rows would hold, estimated for a pyramid that halves
+// from level to level (the level shapes live in device memory): the last level has nk*3/(4^nl - 1) pixels.
+int64_t estimated_cached_rows(const Dims& d, int64_t cap_rows)
+{
+    double last = (double)d.nk;
+    if (d.nl > 1) last = (double)d.nk * 3.0 / ((double)(int64_t(1) << (2 * (d.nl < 16 ? d.nl : 16))) - 1.0);
+    double r = last * 1.1, total = 0.0;
+    for (int l = 0; l < d.nl && total + r <= (double)cap_rows; ++l) {
+        total += r;
+        r *= 4.0;
+    }
+    return (int64_t)total;
+}
+
+// The forward's one-workgroup-per-CU form (msda_fwd_cu.hip): whether a problem takes it, and its launch geometry.
+// It needs 16-byte lanes, rows of at most 16 lanes and the plain operator; it pays when at least the last level fits
+// the CU's LDS and the problem is large enough to keep 256 such workgroups busy well beyond their cache fill.
+bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_msda_plan* p, int* cache_bytes)
+{
+    const int mode = tuning().fwd_cu;
+    const int es = elem_size(dtype);
+    if (mode == 0 || vec * es != 16 || npass != 1 || lpr > 16) return false;
+    const int cap = mxd::kCuLdsBytes - mxd::kCuTableBytes;  // (two level tables come first)
+    const int64_t cap_rows = cap / (d.hd * es) - 1;
+    const int64_t cached = estimated_cached_rows(d, cap_rows);
+    if (mode < 0 && (cached == 0 || d.bs * d.nh * d.nq * d.nl * d.np < (int64_t(1) << 20))) return false;
+    const int U = mxd::kWave / lpr;
+    const int64_t groups = (d.nq + U - 1) / U;
+    // Workgroups per (batch, head): every XCD has 32 CUs, each of which runs one workgroup at a time; the launch
+    // lasts (rounds of 32 workgroups per XCD) x (cache fill + the workgroup's share of the gathers).  The rows that
+    // are not cached come from the XCD's 4 MiB L2: the workgroups that run side by side on an XCD should work on as
+    // few (batch, head) slices as possible (workgroups of an XCD are numbered head, query range, batch element).
+    int64_t best_p = 1;
+    double best_cost = -1.0;
+    const int64_t max_p = groups < 512 ? groups : 512;
+    const double slice_bytes = (double)(d.nk - cached) * (double)(d.hd * es);
+    for (int64_t P = 1; P <= max_p; ++P) {
+        if (tuning().fwd_cu_wgs > 0 && P != tuning().fwd_cu_wgs && tuning().fwd_cu_wgs <= max_p) continue;
+        const int64_t tq = U * (((d.nq + P - 1) / P + U - 1) / U);
+        const int64_t nt = (d.nq + tq - 1) / tq;
+        mxd_msda_plan trial;
+        memset(&trial, 0, sizeof(trial));
+        const int64_t grid = fill_xcd_map(&trial, d.bs, d.nh, nt);
+        const double per_xcd = (double)grid / mxd::kNumXcd;
+        const double rounds = ceil(per_xcd / 32.0);
+        double slices = 32.0 / (double)(trial.xcd_mode == 2 ? trial.tiles_per_part : nt);  // side by side on an XCD
+        if (trial.xcd_mode == 1 && slices < (double)trial.heads_per_xcd) slices = (double)trial.heads_per_xcd;
+        if (trial.xcd_mode == 0) slices = slices * 8.0 < (double)d.nh ? (double)d.nh : slices * 8.0;
+        if (slices < 1.0) slices = 1.0;
+        double over = ceil(slices) * slice_bytes / (4.0 * 1024 * 1024) - 0.8;
+        over = over < 0.0 ? 0.0 : (over > 1.0 ? 1.0 : over);
+        const double cost = rounds * ((double)cached + 3000.0 + (1.0 + 0.5 * over) * (double)tq * (double)(d.nl * d.np) * 4.0);
+        if (best_cost < 0.0 || cost < best_cost) {
+            best_cost = cost;
+            best_p = P;
+        }
+    }
+    const int64_t tq = U * (((d.nq + best_p - 1) / best_p + U - 1) / U);
+    const int64_t nt = (d.nq + tq - 1) / tq;
+    memset(p, 0, sizeof(*p));
+    p->vec = vec;
+    p->lanes_per_row = lpr;
+    p->npass = 1;
+    p->units_per_wave = U;
+    p->waves_per_block = mxd::kCuWaves;
+    p->iters = (int32_t)((tq / U + mxd::kCuWaves - 1) / mxd::kCuWaves);
+    p->tile_q = (int32_t)tq;
+    const int64_t grid = fill_xcd_map(p, d.bs, d.nh, nt);
+    if (grid >= (int64_t(1) << 31)) return false;
+    p->grid = (uint32_t)grid;
+    p->block = (uint32_t)(mxd::kCuWaves * mxd::kWave);
+    p->lds_bytes = (uint32_t)mxd::kCuLdsBytes;
+    *cache_bytes = cap & ~15;
+    return true;
+}
+
 // level_cache: in/out, bytes of LDS for the forward's level cache (asked for -> granted)
-int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_plan* p, int* level_cache = nullptr)
+// cu_form: in/out, whether the forward may take / takes the one-workgroup-per-CU form
+int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_plan* p, int* level_cache = nullptr,
+              int* cu_form = nullptr)
 {
     const int rc = check_dims(dtype, d);
     if (rc != MXD_OK) return rc;
     const int es = elem_size(dtype);
-    if (align_bytes < es) align_bytes = es;
-    int vec = 16 / es;
-    while (vec > 1 && (d.hd % vec != 0 || align_bytes < vec * es)) vec >>= 1;
-    const int lanes_needed = (int)((d.hd + vec - 1) / vec);
-    int lpr = 4;
-    while (lpr < lanes_needed && lpr < mxd::kWave) lpr <<= 1;
-    int npass = (lanes_needed + lpr - 1) / lpr;
-    if (npass == 3) npass = 4;
+    int vec, lpr, npass;
+    row_geometry(es, d.hd, align_bytes, &vec, &lpr, &npass);
+    if (!backward && cu_form && *cu_form && level_cache) {
+        if (plan_forward_cu(dtype, d, vec, lpr, npass, p, level_cache)) return MXD_OK;
+    }
+    if (cu_form) *cu_form = 0;
     memset(p, 0, sizeof(*p));
     p->vec = vec;
     p->lanes_per_row = lpr;
     p->npass = npass;
     p->units_per_wave = mxd::kWave / lpr;
     p->waves_per_block = 4;
-    int iters = env_int("MXD_MSDA_FWD_ITERS", 1);
+    int iters = tuning().fwd_iters;
     if (iters < 1) iters = 1;
     const BwdLayout L = bwd_layout(dtype, d);
     // the tile pass wants L.tile_q queries per workgroup of the first backward kernel
@@ -277,7 +453,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
             waves >>= 1;
         if (waves > 2) {
             p->waves_per_block = waves;
-            iters = env_int("MXD_MSDA_FWD_WGQ", 128) / (p->units_per_wave * p->waves_per_block);
+            iters = tuning().fwd_wgq / (p->units_per_wave * p->waves_per_block);
             if (iters < 1) iters = 1;
         } else {
             cache = 0;
@@ -291,11 +467,13 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     if (grid >= (int64_t(1) << 31)) return fail(MXD_E_SHAPE, "problem needs %lld workgroups, beyond the launch limit", (long long)grid);
     p->grid = (uint32_t)grid;
     p->block = (uint32_t)(p->waves_per_block * mxd::kWave);
-    size_t per_unit = mxd::kChunkStride * sizeof(mxd::Entry);
-    if (backward) per_unit += mxd::kChunk * sizeof(mxd::f32x4);
-    p->lds_bytes = (uint32_t)(mxd::kMaxLevels * sizeof(mxd::i32x4) + (size_t)p->waves_per_block * p->units_per_wave * per_unit);
-    if (backward && L.tiles) p->lds_bytes += (uint32_t)((mxd::kMaxLevels + L.tbl_stride) * sizeof(int32_t));
-    if (!backward) p->lds_bytes += (uint32_t)(p->waves_per_block * p->units_per_wave * 2 * sizeof(float));  // softmax statistics (fused form)
+    if (backward) {
+        p->lds_bytes = (uint32_t)backward_lds_bytes(p->units_per_wave, p->waves_per_block, L.tiles, L.tbl_stride);
+    } else {
+        p->lds_bytes = (uint32_t)(mxd::kMaxLevels * sizeof(mxd::i32x4) +
+                                  (size_t)p->waves_per_block * p->units_per_wave * mxd::kChunkStride * sizeof(mxd::Entry));
+        p->lds_bytes += (uint32_t)(p->waves_per_block * p->units_per_wave * 2 * sizeof(float));  // softmax statistics (fused form)
+    }
     if (cache > 0) p->lds_bytes += (uint32_t)cache;
     if (level_cache) *level_cache = cache;
     return MXD_OK;
@@ -374,9 +552,17 @@ int mxd_msda_make_plan(int backward, int dtype, int64_t bs, int64_t nk, int64_t 
     take_meta_flag(&dtype);
     if (!plan) return fail(MXD_E_NULL, "plan is NULL");
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
-    int cache = 1;
-    return make_plan(backward != 0, dtype, d, align_bytes, plan, &cache);
+    int cache = 1, cu = 1;
+    return make_plan(backward != 0, dtype, d, align_bytes, plan, &cache, &cu);
 }
+
+int mxd_msda_init(void)
+{
+    tuning();
+    return ensure_device_ready();
+}
+
+void mxd_msda_reload_tuning(void) { tuning(); read_tuning(); }
 
 int mxd_msda_decode_block(const mxd_msda_plan* plan, uint32_t block_index, int64_t bs, int64_t nh, int64_t nq,
                           int32_t work[4])
@@ -409,8 +595,12 @@ static int forward_common(int kind, const void* value, const int32_t* spatial_sh
     if (ptr_align(output) < align) align = ptr_align(output);
     mxd::KArgs a;
     memset(&a, 0, sizeof(a));
+    rc = ensure_device_ready();
+    if (rc != MXD_OK) return rc;
     int cache = kind == 0;
-    rc = make_plan(0, dtype, d, align, &a.plan, &cache);
+    // (the one-workgroup-per-CU form reads a location pair with one load)
+    int cu = kind == 0 && ptr_align(sampling_loc) >= 2 * elem_size(dtype);
+    rc = make_plan(0, dtype, d, align, &a.plan, &cache, &cu);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
     a.meta_i64 = meta64;
@@ -425,8 +615,9 @@ static int forward_common(int kind, const void* value, const int32_t* spatial_sh
     a.grid_h = (int32_t)grid_h;
     a.grid_w = (int32_t)grid_w;
     a.lds_cache_bytes = cache;
-    a.fwd_ahead = env_int("MXD_MSDA_FWD_AHEAD", 1);
-    const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
+    a.fwd_ahead = tuning().fwd_ahead;
+    const hipError_t e = cu ? mxd::launch_forward_cu(dtype, a, static_cast<hipStream_t>(hip_stream))
+                            : mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(e));
     return MXD_OK;
 }
@@ -596,25 +787,28 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     }
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * nk * nh * hd;
+    // every step that can fail for the sizes given comes before the first launch
+    const bool atomic_mode = !L.tiles;
+    mxd::TileArgs t;
+    if (!atomic_mode) {
+        rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
+        if (rc != MXD_OK) return rc;
+        t.store_vec = (hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
+    }
     hipError_t e = hipSuccess;
     // zero-fill of the image: by the first kernel's workgroups when the tile pass is the first to touch it and it
     // can be written in 16-byte pieces, by a kernel of its own otherwise
     const bool fill_inside = L.tiles && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 &&
-                             env_int("MXD_MSDA_BWD_FILL_KERNEL", 0) == 0;
+                             tuning().bwd_fill_kernel == 0;
     if (!(flags & MXD_BWD_ACCUMULATE)) {
         if (fill_inside) a.fill_n4 = n / 4;
         else e = mxd::launch_fill_zero(image, n, stream);
     }
     if (e == hipSuccess && part && !a.np_pow2) e = mxd::launch_fill_zero(part, part_bytes / sizeof(float), stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: zero-fill launch failed: %s", who, hipGetErrorString(e));
-    const bool atomic_mode = !L.tiles;
     e = mxd::launch_backward(dtype, a, atomic_mode, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(e));
     if (!atomic_mode) {
-        mxd::TileArgs t;
-        rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
-        if (rc != MXD_OK) return rc;
-        t.store_vec = (hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
         e = mxd::launch_gradv_tiles(dtype, a, t, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: tile kernel launch failed: %s", who, hipGetErrorString(e));
     }
@@ -794,21 +988,24 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     a.grad_attn = grad_weights;
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * num_feat * num_embeds;
+    // every step that can fail for the sizes given comes before the first launch
+    const bool atomic_mode = !L.tiles;
+    mxd::TileArgs t;
+    if (!atomic_mode) {
+        rc = make_tile_args(d, L, a.plan.vec, 0, &t);
+        if (rc != MXD_OK) return rc;
+        t.store_vec = (d.hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
+    }
     hipError_t e = hipSuccess;
-    if (L.tiles && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 && env_int("MXD_MSDA_BWD_FILL_KERNEL", 0) == 0)
+    if (L.tiles && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 && tuning().bwd_fill_kernel == 0)
         a.fill_n4 = n / 4;  // zero-filled by the first kernel's workgroups
     else
         e = mxd::launch_fill_zero(image, n, stream);
     if (e == hipSuccess && !a.sc_pow2) e = mxd::launch_fill_zero(part, part_bytes / sizeof(float), stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: zero-fill launch failed: %s", hipGetErrorString(e));
-    const bool atomic_mode = !L.tiles;
     e = mxd::launch_backward(dtype, a, atomic_mode, stream);
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: launch failed: %s", hipGetErrorString(e));
     if (!atomic_mode) {
-        mxd::TileArgs t;
-        rc = make_tile_args(d, L, a.plan.vec, 0, &t);
-        if (rc != MXD_OK) return rc;
-        t.store_vec = (d.hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
         e = mxd::launch_gradv_tiles(dtype, a, t, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: tile kernel launch failed: %s", hipGetErrorString(e));
     }

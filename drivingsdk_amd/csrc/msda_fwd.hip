@@ -306,26 +306,12 @@ static hipError_t launch_one(const KArgs& a, hipStream_t stream)
         hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcDagg, false>), grid, block, a.plan.lds_bytes, stream, a);
     else if (a.ref != nullptr)
         hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcFused, false>), grid, block, a.plan.lds_bytes, stream, a);
-    else if (a.ref != nullptr)
-        hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcFused, false>), grid, block, a.plan.lds_bytes, stream, a);
     else {
         // look-ahead form: one chunk of samples per unit and at most two samples per lane
         const bool ahead = a.fwd_ahead != 0 && a.S <= kChunk && a.plan.units_per_wave * kChunk <= 2 * kWave;
         if (a.lds_cache_bytes > 0) {
+            // (more than the 64 KiB of dynamic LDS a kernel gets by default: raise_forward_lds() has opted in)
             if constexpr (VEC * sizeof(T) == 16) {
-                // more than the 64 KiB of dynamic LDS a kernel gets by default: opt in once per instantiation
-                static bool raised = false;
-                if (!raised) {
-                    hipError_t e = hipFuncSetAttribute(
-                        reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, false>),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-                    if (e == hipSuccess)
-                        e = hipFuncSetAttribute(
-                            reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, true>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-                    if (e != hipSuccess) return e;
-                    raised = true;
-                }
                 if (ahead)
                     hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, true>), grid, block, a.plan.lds_bytes, stream, a);
                 else
@@ -339,6 +325,26 @@ static hipError_t launch_one(const KArgs& a, hipStream_t stream)
             hipLaunchKernelGGL((msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, false, false>), grid, block, a.plan.lds_bytes, stream, a);
     }
     return hipGetLastError();
+}
+
+// The level-cache instantiations use up to 80 KiB of dynamic LDS: opt in, on the current device.
+template <typename T, int VEC, int NPASS>
+static hipError_t raise_one()
+{
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_kernel<T, VEC, NPASS, kSrcPlain, true, true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+    return e;
+}
+
+hipError_t raise_forward_lds()
+{
+    hipError_t e = raise_one<float, 4, 1>();
+    if (e == hipSuccess) e = raise_one<f16_t, 8, 1>();
+    if (e == hipSuccess) e = raise_one<bf16_t, 8, 1>();
+    return e;
 }
 
 template <typename T>

@@ -29,6 +29,11 @@ constexpr int kMaxLevels = 64;
 constexpr int kChunk = 16;           // samples of a unit staged per pass
 constexpr int kChunkStride = 17;     // staged entries per unit incl. one pad entry (LDS banks)
 
+// Dynamic LDS of the forward's one-workgroup-per-CU form: the whole LDS of a gfx950 CU.
+constexpr int kCuLdsBytes = 160 * 1024;
+constexpr int kCuWaves = 16;         // wavefronts of its workgroups
+constexpr int kCuTableBytes = 2 * (kMaxLevels + 1) * 16 + 32;  // its two level tables ahead of the cached rows (multiple of 64)
+
 constexpr int kTilePx = 512;         // pixels per tile of the grad_value pass = threads of its workgroups
 constexpr int kTilePxLog2 = 9;
 

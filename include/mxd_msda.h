@@ -19,7 +19,9 @@
  *     CURRENT device and the call returns without synchronising.
  *   - Return value: 0 on success, a negative MXD_E_* code otherwise; the message for the
  *     calling thread's last failure is returned by mxd_msda_last_error().
- *   - Thread safe: no mutable global state except the thread-local error message.
+ *   - Thread safe.  Process-wide state: the tuning knobs (MXD_MSDA_* environment variables, read once on first
+ *     use), one "set up" flag per device (the first call on a device opts its large-LDS kernels in; mxd_msda_init()
+ *     does the same ahead of time), and the thread-local error message.
  *
  * Layouts (T = element type selected by `dtype`)
  *   value            T   [bs, nk, nh, hd]
@@ -96,6 +98,16 @@ int mxd_msda_version(void);
 
 /* Message of the calling thread's most recent failed call ("" if none). */
 const char* mxd_msda_last_error(void);
+
+/* Optional.  Does, for the CURRENT device, the one-time set-up that the compute entry points otherwise do on their
+ * first call there (function attributes of the kernels that use more than 64 KiB of LDS): call it once per device
+ * before capturing the library's launches in a HIP graph without a warm-up call.  Returns 0 or MXD_E_LAUNCH.
+ * No counterpart in the reference (its launcher resolves its symbols lazily, include/csrc/OpApiCommon.h:117-132). */
+int mxd_msda_init(void);
+
+/* Reads the MXD_MSDA_* tuning variables from the environment again (they are otherwise read once per process).
+ * A hook for tests and experiments; must not run while another thread is inside the library. */
+void mxd_msda_reload_tuning(void);
 
 /* Compute the launch geometry for a problem without touching the GPU.
  * `backward` = 0/1.  `align_bytes` = the largest power of two (<= 16) dividing every data

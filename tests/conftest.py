@@ -38,3 +38,13 @@ def gpu_device():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda", 0)
+
+
+@pytest.fixture(autouse=True)
+def _tuning_follows_the_environment():
+    """The library reads its MXD_MSDA_* tuning variables once per process; tests that change them call
+    util.set_tuning(), and after every test (monkeypatch has restored the environment by then) they are read again."""
+    yield
+    from drivingsdk_amd import _lib
+    if _lib._lib is not None:
+        _lib.reload_tuning()

@@ -55,8 +55,16 @@ def test_plan_covers_every_unit_exactly_once(backward, dims):
         assert plan.vec * plan.lanes_per_row * plan.npass >= hd
         assert hd % plan.vec == 0
         assert plan.block == 64 * plan.waves_per_block
-        assert plan.tile_q == plan.units_per_wave * plan.waves_per_block * plan.iters
-        assert plan.lds_bytes <= 80 * 1024   # two workgroups per CU
+        if plan.block == 1024:
+            # the forward's one-workgroup-per-CU form: a workgroup takes a whole CU's LDS and any multiple of
+            # units_per_wave queries, its wavefronts taking groups of units_per_wave in turn
+            assert not backward and plan.lds_bytes == 160 * 1024
+            assert plan.tile_q % plan.units_per_wave == 0
+            assert plan.tile_q <= plan.units_per_wave * plan.waves_per_block * plan.iters
+        else:
+            assert plan.tile_q == plan.units_per_wave * plan.waves_per_block * plan.iters
+            # two workgroups per CU (forward), the default dynamic LDS limit (backward)
+            assert plan.lds_bytes <= (64 if backward else 80) * 1024
         seen = {}
         work = (ctypes.c_int32 * 4)()
         for bid in range(plan.grid):

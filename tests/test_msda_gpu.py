@@ -10,7 +10,7 @@ import torch
 
 from drivingsdk_amd import _lib, workloads
 from oracle import msda_oracle as orc
-from util import BWD_FP32, FWD_FP32, HALF, oracle_all, rel_err, run_gpu, to_device
+from util import BWD_FP32, FWD_FP32, HALF, oracle_all, rel_err, run_gpu, set_tuning, to_device
 
 pytestmark = pytest.mark.gpu
 
@@ -474,8 +474,7 @@ def test_backward_launch_variants_agree_with_the_oracle(gpu_device, monkeypatch,
     """The tuning knobs read at call time select other code paths (one-kernel atomic backward, other
     workgroup sizes of the first kernel, tiles split into very many or no query chunks, plain workgroup
     mapping, zero-fill by a kernel of its own); every one of them must give the same gradients."""
-    for k, v in env.items():
-        monkeypatch.setenv(k, v)
+    set_tuning(monkeypatch, **env)
     for name, scale in (("tiny", 1.0), ("detr_encoder_bwd", 0.25)):
         inp = workloads.make_inputs(name, with_grad_output=True, scale_queries=scale)
         errs = _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
@@ -487,7 +486,7 @@ def test_backward_launch_variants_agree_with_the_oracle(gpu_device, monkeypatch,
 def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
     """The forward's level cache (rows of the last levels held in LDS) is switched by an estimate of the level
     sizes; here it is forced off and on with room for no, one, several and all levels, for every dtype."""
-    monkeypatch.setenv("MXD_MSDA_FWD_LDS", lds)
+    set_tuning(monkeypatch, MXD_MSDA_FWD_LDS=lds, MXD_MSDA_FWD_CU=0)   # (the general forward kernel's cache)
     tol = FWD_FP32 if dtype == torch.float32 else (HALF if dtype == torch.float16 else 2.0 ** -8)
     for name, scale in (("tiny", 1.0), ("detr_encoder", 0.1)):
         inp = workloads.make_inputs(name, dtype=dtype, scale_queries=scale)
@@ -498,21 +497,25 @@ def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
 
 @pytest.mark.parametrize("env", [{"MXD_MSDA_FWD_AHEAD": "0"}, {"MXD_MSDA_FWD_AHEAD": "0", "MXD_MSDA_FWD_LDS": "0"},
                                  {"MXD_MSDA_FWD_LDS": "0"}, {"MXD_MSDA_FWD_WGQ": "64"}, {"MXD_MSDA_FWD_WGQ": "512"},
-                                 {"MXD_MSDA_FWD_LDS": "0", "MXD_MSDA_FWD_ITERS": "3"}],
+                                 {"MXD_MSDA_FWD_LDS": "0", "MXD_MSDA_FWD_ITERS": "3"},
+                                 {"MXD_MSDA_FWD_CU": "1"}, {"MXD_MSDA_FWD_CU": "1", "MXD_MSDA_FWD_CU_WGS": "3"},
+                                 {"MXD_MSDA_FWD_CU": "1", "MXD_MSDA_FWD_CU_WGS": "500"}],
                          ids=lambda e: ",".join(f"{k[9:]}={v}" for k, v in e.items()))
 def test_forward_launch_variants_agree(gpu_device, monkeypatch, env):
     """The forward requests the samples of a wavefront's next units ahead of the gather of the current ones (with and
-    without the level cache, one or several iterations per wavefront, the last one partly filled); every such
-    launch form must give the same output, bit for bit, as the form without it, and meet the oracle."""
+    without the level cache, one or several iterations per wavefront, the last one partly filled), and for large
+    problems it runs as one workgroup per CU with the last levels in LDS (forced here for small ones, with few and
+    with very many workgroups per (batch, head)); every such launch form must give the same output, bit for bit,
+    as the form without it, and meet the oracle."""
     for name, scale in (("tiny", 1.0), ("detr_encoder", 0.13), ("bevformer_sca", 0.03)):  # (the last: 32 samples per unit)
         inp = workloads.make_inputs(name, scale_queries=scale)
         want = oracle_all(inp, with_grads=False)[0]
         base = run_gpu(inp, gpu_device, with_grads=False)[0]
         assert rel_err(base, want) <= FWD_FP32, name
         with monkeypatch.context() as m:
-            for k, v in env.items():
-                m.setenv(k, v)
+            set_tuning(m, **env)
             got = run_gpu(inp, gpu_device, with_grads=False)[0]
+        _lib.reload_tuning()   # (the context has restored the environment)
         assert np.array_equal(np.asarray(got), np.asarray(base)), (name, env)
 
 
@@ -572,7 +575,7 @@ def test_hot_pixels_get_extra_lists_in_the_tile_pass(gpu_device, monkeypatch, le
     samples go to three spots of the first level (one of them in its last, partial tile), the others are
     uniform, and a large work-item size keeps every tile in one work item, so that the rounds after the first
     run with extra lists, pair entries among the moved ones."""
-    monkeypatch.setenv("MXD_MSDA_TILE_TARGET", "1000000")
+    set_tuning(monkeypatch, MXD_MSDA_TILE_TARGET=1000000)
     g = torch.Generator().manual_seed(11)
     shapes, lsi = workloads.level_tensors(levels)
     nk = int(shapes.prod(1).sum())
@@ -597,7 +600,7 @@ def test_random_hot_spots_many_rounds(gpu_device, monkeypatch, seed):
     head sizes, float32 and float16; with the default work-item size for even seeds and unsplit tiles for odd ones."""
     rng = np.random.default_rng(100 + seed)
     if seed % 2:
-        monkeypatch.setenv("MXD_MSDA_TILE_TARGET", "1000000")
+        set_tuning(monkeypatch, MXD_MSDA_TILE_TARGET=1000000)
     nl = int(rng.integers(1, 4))
     levels = [(int(rng.integers(3, 40)), int(rng.integers(3, 40))) for _ in range(nl)]
     shapes, lsi = workloads.level_tensors(levels)
@@ -673,3 +676,58 @@ def test_random_small_problems_16bit(gpu_device, seed):
         if name == "grad_sampling_locations":
             g_, r_ = g_ * keep, r_ * keep
         assert rel_err(g_, r_) <= tol, (name, rel_err(g_, r_), desc)
+
+
+@pytest.mark.parametrize("name,dtype", [("detr_encoder", torch.float32), ("detr_encoder", torch.float16),
+                                        ("detr_encoder", torch.bfloat16), ("bevformer_sca", torch.float32),
+                                        ("bevformer_sca", torch.float16), ("head_dim_128", torch.float16),
+                                        ("head_dim_128", torch.bfloat16)])
+def test_forward_cu_form_equals_the_general_form_at_full_size(gpu_device, monkeypatch, name, dtype):
+    """The benchmark shapes take the forward's one-workgroup-per-CU form by default (last levels in LDS, sample values
+    handed across lanes by DPP; rows of 8, 4 and 16 lanes here).  Its sums run in the same order as the general
+    kernel's, so at full size the two must agree bit for bit; the general kernel is checked against the oracle at these
+    sizes elsewhere."""
+    from drivingsdk_amd import _C
+    d = to_device(workloads.make_inputs(name, dtype=dtype), gpu_device)
+    args = (d.value, d.spatial_shapes, d.level_start_index, d.sampling_locations, d.attention_weights)
+    plan = _lib.make_plan(0, {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype], *d.value.shape,
+                          d.spatial_shapes.shape[0], d.spatial_shapes.shape[0], d.sampling_locations.shape[1],
+                          d.sampling_locations.shape[4])
+    assert plan.block == 1024, "the benchmark shapes are meant to take the one-workgroup-per-CU form"
+    out_cu = _C.multi_scale_deformable_attn(*args)
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=0)
+    out_general = _C.multi_scale_deformable_attn(*args)
+    assert torch.equal(out_cu, out_general)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_small_problems_cu_form(gpu_device, monkeypatch, seed):
+    """Random small problems forced through the one-workgroup-per-CU forward wherever it can run (16-byte lanes, rows
+    of at most 16 lanes): odd point counts (the sample-by-sample path), level lists that end inside a chunk, levels
+    that do and do not fit the LDS, float32 and 16-bit storage; against the oracle."""
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=1, MXD_MSDA_FWD_CU_WGS=1 + seed % 5)
+    rng = np.random.default_rng(3000 + seed)
+    dtype = (torch.float32, torch.float16, torch.bfloat16)[seed % 3]
+    es = 4 if dtype == torch.float32 else 2
+    bs, nq, nh = int(rng.integers(1, 4)), int(rng.integers(1, 900)), int(rng.integers(1, 10))
+    hd = int(rng.choice([4, 8, 12, 16, 24, 32, 48, 64])) * (16 // es) // 4   # rows of 16 .. 256 bytes, multiples of 16
+    nl, npts = int(rng.integers(1, 6)), int(rng.integers(1, 10))
+    big = seed % 4 == 0   # a first level that cannot fit the LDS (1 350 rows of up to 256 bytes ...), small ones behind it
+    levels = [(int(rng.integers(1, 48)), int(rng.integers(1, 48))) for _ in range(nl)]
+    if big:
+        levels[0] = (90, 150)
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    g = torch.Generator().manual_seed(3000 + seed)
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g).to(dtype), shapes, lsi,
+                               (torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.3 - 0.15).to(dtype),
+                               torch.rand(bs, nq, nh, nl, npts, generator=g).to(dtype), None)
+    print("case", (bs, nq, nh, hd, levels, npts), dtype, flush=True)
+    want = oracle_all(inp, with_grads=False)[0]
+    got = run_gpu(inp, gpu_device, with_grads=False)[0]
+    tol = FWD_FP32 if dtype == torch.float32 else (HALF if dtype == torch.float16 else 2.0 ** -8)
+    assert rel_err(got, want) <= tol
+    with monkeypatch.context() as m:
+        set_tuning(m, MXD_MSDA_FWD_CU=0)
+        general = run_gpu(inp, gpu_device, with_grads=False)[0]
+    assert np.array_equal(np.asarray(got), np.asarray(general))

@@ -55,3 +55,12 @@ def run_gpu(inp, device, with_grads=True):
         res += [None, None, None]
     torch.cuda.synchronize()
     return res
+
+
+def set_tuning(monkeypatch, **env):
+    """Set MXD_MSDA_* tuning variables for the rest of a test and have the library read them (it reads the
+    environment once per process otherwise; conftest reads it again after the test)."""
+    from drivingsdk_amd import _lib
+    for k, v in env.items():
+        monkeypatch.setenv(k, str(v))
+    _lib.reload_tuning()
