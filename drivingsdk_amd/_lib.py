@@ -27,6 +27,8 @@ EXPORTS = (
     "mxd_msda_fused_backward",
     "mxd_msda_backward_workspace_bytes",
     "mxd_msda_backward",
+    "mxd_msda_backward_static_limit",
+    "mxd_msda_backward_static",
     "mxd_dagg_forward",
     "mxd_dagg_backward_workspace_bytes",
     "mxd_dagg_backward",
@@ -91,6 +93,10 @@ def load():
     lib.mxd_msda_backward_workspace_bytes.argtypes = [ci] + [i64] * 8
     lib.mxd_msda_backward.restype = ci
     lib.mxd_msda_backward.argtypes = [p] * 10 + [ctypes.c_size_t, ci] + [i64] * 8 + [ci, p]
+    lib.mxd_msda_backward_static_limit.restype = ctypes.c_size_t
+    lib.mxd_msda_backward_static_limit.argtypes = []
+    lib.mxd_msda_backward_static.restype = ci
+    lib.mxd_msda_backward_static.argtypes = [p] * 9 + [ci] + [i64] * 8 + [ci, p]
     lib.mxd_dagg_forward.restype = ci
     lib.mxd_dagg_forward.argtypes = [p] * 6 + [ci] + [i64] * 8 + [p]
     lib.mxd_dagg_backward_workspace_bytes.restype = ctypes.c_size_t

@@ -105,10 +105,18 @@ const Tuning& tuning()
     return g_tuning;
 }
 
+// Scratch of mxd_msda_backward_static(): the hand-over between the two backward kernels (and the fp32 image of
+// grad_value for 16-bit dtypes) for callers that can neither allocate nor pass a workspace.  Every device that the
+// library runs on holds its own copy of the array at its own address until the process ends.  In host code the name
+// below is a stand-in, not a device address: g_scratch_ptr[device], resolved once per device, is what is used.
+constexpr size_t kStaticScratchBytes = (size_t)MXD_MSDA_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 // Per-device set-up, done once per device on the first call that needs it (or by mxd_msda_init()): the forward
-// kernels that use more than 64 KiB of dynamic LDS opt in.
+// kernels that use more than 64 KiB of dynamic LDS opt in, and the device address of `scratch` is looked up.
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_device_ready[kMaxDevices];
+void* g_scratch_ptr[kMaxDevices];
 std::mutex g_device_mutex;
 
 int ensure_device_ready()
@@ -123,8 +131,21 @@ int ensure_device_ready()
     e = mxd::raise_forward_lds();
     if (e == hipSuccess) e = mxd::raise_forward_cu_lds();
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "raising the dynamic LDS limit failed: %s", hipGetErrorString(e));
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));  // (this device's copy of the array: the device is current)
+    if (e != hipSuccess || ptr == nullptr)
+        return fail(MXD_E_LAUNCH, "looking up the static scratch array failed: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
     g_device_ready[dev].store(1, std::memory_order_release);
     return MXD_OK;
+}
+
+// The current device's copy of `scratch` (after ensure_device_ready()).
+void* device_scratch()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    return g_device_ready[dev].load(std::memory_order_acquire) ? g_scratch_ptr[dev] : nullptr;
 }
 
 struct Dims {
@@ -854,6 +875,30 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
     return backward_common(0, value, spatial_shapes, level_start_index, sampling_loc, attn_weight, grad_output,
                            grad_value, grad_loc, grad_attn, workspace, workspace_bytes, dtype, bs, nk, nh, hd, nl,
                            nl_attn, nq, np, flags, hip_stream);
+}
+
+size_t mxd_msda_backward_static_limit(void) { return kStaticScratchBytes; }
+
+int mxd_msda_backward_static(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                             const void* sampling_loc, const void* attn_weight, const void* grad_output,
+                             void* grad_value, void* grad_loc, void* grad_attn, int dtype, int64_t bs, int64_t nk,
+                             int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np, int flags,
+                             void* hip_stream)
+{
+    // (allocates nothing: the scratch is the library's own static device array; sizes beyond it are refused)
+    const size_t need = mxd_msda_backward_workspace_bytes(dtype, bs, nk, nh, hd, nl, nl_attn, nq, np);
+    if (need > kStaticScratchBytes)
+        return fail(MXD_E_WORKSPACE,
+                    "mxd_msda_backward_static: this problem needs %zu bytes of scratch, the static array holds %zu; "
+                    "use mxd_msda_backward with a workspace",
+                    need, kStaticScratchBytes);
+    int rc = ensure_device_ready();
+    if (rc != MXD_OK) return rc;
+    void* ws = device_scratch();
+    if (!ws) return fail(MXD_E_LAUNCH, "mxd_msda_backward_static: the static scratch array is not set up on this device");
+    return backward_common(0, value, spatial_shapes, level_start_index, sampling_loc, attn_weight, grad_output,
+                           grad_value, grad_loc, grad_attn, ws, kStaticScratchBytes, dtype, bs, nk, nh, hd, nl, nl_attn,
+                           nq, np, flags, hip_stream);
 }
 
 size_t mxd_gka_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl,

@@ -193,6 +193,22 @@ int mxd_msda_backward(const void* value, const int32_t* spatial_shapes, const in
                       int64_t bs, int64_t nk, int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq,
                       int64_t np, int flags, void* hip_stream);
 
+/* Backward without a workspace argument and without any allocation.  No counterpart in the reference: it is for
+ * callers that can neither call hipMalloc nor hand over scratch memory -- code under HIP graph capture, tight serving
+ * loops, harnesses that forbid allocation.  It is mxd_msda_backward with the hand-over between its kernels (and the
+ * fp32 image for 16-bit dtypes) in a static device array of MXD_MSDA_STATIC_SCRATCH_BYTES that every GPU the library
+ * runs on holds until the process ends.  Problems whose mxd_msda_backward_workspace_bytes() exceeds that size are
+ * refused with MXD_E_WORKSPACE.  All calls on one GPU share the array: calls that overlap in time on one GPU (other
+ * streams, other threads) race; calls on one stream do not.  Nothing in the array has to survive between calls or
+ * start at zero (the image is zero-filled by the call itself).  mxd_msda_backward_static_limit() returns the size. */
+#define MXD_MSDA_STATIC_SCRATCH_BYTES (32u << 20)
+size_t mxd_msda_backward_static_limit(void);
+int mxd_msda_backward_static(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
+                             const void* sampling_loc, const void* attn_weight, const void* grad_output,
+                             void* grad_value, void* grad_loc, void* grad_attn, int dtype, int64_t bs, int64_t nk,
+                             int64_t nh, int64_t hd, int64_t nl, int64_t nl_attn, int64_t nq, int64_t np, int flags,
+                             void* hip_stream);
+
 /* ---- deformable aggregation (Sparse4D / SparseDrive feature sampling) ------------------------
  * Replaces deformable_aggregation / deformable_aggregation_backward
  * (mx_driving/csrc/DeformableAggregation.cpp:20-82) with the same tensors:
