@@ -350,7 +350,8 @@ def geometric_kernel_attention_forward(value_map, spatial_shapes, level_start_in
            "output: expected a contiguous [bs, num_queries, num_heads*dim] tensor of value's dtype")
     value = value_map.contiguous()
     shapes, lsi = spatial_shapes.int().contiguous(), level_start_index.int().contiguous()
-    loc, attn = sampling_locations.to(dt).contiguous(), attention_weights.to(dt).contiguous()
+    # (pixel indices travel as float32 whatever value's dtype is: exact below 2^24, where a 16-bit float is not)
+    loc, attn = sampling_locations.to(torch.float32).contiguous(), attention_weights.to(dt).contiguous()
     with torch.cuda.device(value.device):
         rc = lib.mxd_gka_forward(value.data_ptr(), shapes.data_ptr(), lsi.data_ptr(), loc.data_ptr(), attn.data_ptr(),
                                  output.data_ptr(), _FLOAT_CODES[dt], *dims, torch.cuda.current_stream().cuda_stream)
@@ -365,8 +366,10 @@ def geometric_kernel_attention_backward(value, spatial_shapes, level_start_index
     lib = _lib.load()
     dt = value.dtype
     value = value.contiguous()
+    _check(grad_output.device == value.device and grad_output.numel() == dims[0] * dims[5] * dims[2] * dims[3],
+           "grad_output: expected [bs, num_queries, num_heads*dim] on value's device")
     shapes, lsi = spatial_shapes.int().contiguous(), level_start_index.int().contiguous()
-    loc, attn = sampling_locations.to(dt).contiguous(), attn_weights.to(dt).contiguous()
+    loc, attn = sampling_locations.to(torch.float32).contiguous(), attn_weights.to(dt).contiguous()
     go = grad_output.to(dt).contiguous()
     gv, ga = torch.empty_like(value), torch.empty_like(attn)
     code = _FLOAT_CODES[dt]
@@ -428,7 +431,10 @@ def grid_sampler2d_v2_backward(grad_output, input_x, input_grid, interpolation_m
            "grid_sampler2d_v2_backward(): all tensors must live on a GPU (this build has no CPU implementation)")
     n, h_in, w_in, c = input_x.shape
     _, h_out, w_out, _ = input_grid.shape
+    _check(input_grid.size(0) == n and input_grid.size(3) == 2, "input_grid: expected [N, H_out, W_out, 2]")
     _check(tuple(grad_output.shape) == (n, h_out, w_out, c), "grad_output: expected [N, H_out, W_out, C]")
+    _check(grad_output.device == input_x.device and input_grid.device == input_x.device,
+           "grid_sampler2d_v2_backward(): tensors are on different devices")
     lib = _lib.load()
     dt = input_x.dtype
     _check(dt in _FLOAT_CODES, f"input_x: float tensor expected but got {dt}")

@@ -83,7 +83,6 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     Entry* stage = reinterpret_cast<Entry*>(strip);
     f32x4* dots = reinterpret_cast<f32x4*>(strip + (size_t)U * kChunkStride * sizeof(Entry));
 
-    const T* loc = static_cast<const T*>(a.loc);
     const T* attn = static_cast<const T*>(a.attn);
     const T* gout = static_cast<const T*>(a.grad_out);
     T* gloc = static_cast<T*>(a.grad_loc);
@@ -191,8 +190,8 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             r.active = (i < entries) && (q < wk.q_end) && (s < a.S);
             if (r.active) {
                 const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
-                r.x = to_f32(loc[2 * sr.loc_e]);
-                r.y = to_f32(loc[2 * sr.loc_e + 1]);
+                r.x = load_coord<SRC, T>(a.loc, 2 * sr.loc_e);
+                r.y = load_coord<SRC, T>(a.loc, 2 * sr.loc_e + 1);
                 if constexpr (SRC == kSrcGrid) r.aw = 1.0f;  // no weights tensor
                 else r.aw = to_f32(attn[sr.w_e]);
                 r.l = sr.l;
@@ -277,7 +276,6 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         }
         for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) cursor[i] = 0;
         __syncthreads();
-        const T* loc0 = static_cast<const T*>(a.loc);
         const int early_units = kEarly ? a.plan.waves_per_block * U : 0;  // their first kChunk samples are counted here:
         if constexpr (kEarly) {
             const int q0 = wk.q_begin + wave * U;
@@ -303,7 +301,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             if (act) {
                 const SampleRef sr = sample_ref<SRC>(a, wk.b, wk.q_begin + qr, wk.h, s);
                 l = sr.l;
-                float cx = to_f32(loc0[2 * sr.loc_e]), cy = to_f32(loc0[2 * sr.loc_e + 1]);
+                float cx = load_coord<SRC, T>(a.loc, 2 * sr.loc_e), cy = load_coord<SRC, T>(a.loc, 2 * sr.loc_e + 1);
                 if constexpr (FUSED)
                     fused_location(a, static_cast<const T*>(a.ref) + (((int64_t)wk.b * a.nq + wk.q_begin + qr) * a.nl + l) * a.ref_dim,
                                    lvl[l], cx, cy);
@@ -496,12 +494,12 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                             sm.w[k] = sm.valid ? wt[k] : 0.0f;
                         }
                         if constexpr (FUSED) {
-                            ox = to_f32(loc[2 * sr.loc_e]);
-                            oy = to_f32(loc[2 * sr.loc_e + 1]);
+                            ox = load_coord<SRC, T>(a.loc, 2 * sr.loc_e);
+                            oy = load_coord<SRC, T>(a.loc, 2 * sr.loc_e + 1);
                         }
                     } else {
-                        float x = to_f32(loc[2 * sr.loc_e]);
-                        float y = to_f32(loc[2 * sr.loc_e + 1]);
+                        float x = load_coord<SRC, T>(a.loc, 2 * sr.loc_e);
+                        float y = load_coord<SRC, T>(a.loc, 2 * sr.loc_e + 1);
                         if constexpr (SRC != kSrcGrid) aw = to_f32(attn[sr.w_e]);
                         ox = x;
                         oy = y;

@@ -162,6 +162,15 @@ __device__ inline T from_f32(float v)
     return (T)v;
 }
 
+// One coordinate of a sampling location.  Geometric kernel attention carries pixel indices: they are float32 whatever
+// the element type of value is (a 16-bit float cannot hold the indices of a level wider than 2048 / 256 pixels).
+template <int SRC, typename T>
+__device__ inline float load_coord(const void* loc, int64_t i)
+{
+    if constexpr (SRC == kSrcGka) return static_cast<const float*>(loc)[i];
+    else return to_f32(static_cast<const T*>(loc)[i]);
+}
+
 // Fused form: sampling location from the raw offset (x, y) of a sample on level `lv` = {H, W, ..}.
 // rp: the query's reference point on that level, (cx, cy) or a box (cx, cy, w, h).
 //   points: location = reference + offset / (W, H)          boxes: location = centre + offset / np * (w, h) / 2

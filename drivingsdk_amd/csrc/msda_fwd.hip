@@ -107,7 +107,6 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
     float* stats = reinterpret_cast<float*>(stage_all + a.plan.waves_per_block * (U * kChunkStride)) + wave * (2 * U);
     const T* ref = static_cast<const T*>(a.ref);
 
-    const T* loc = static_cast<const T*>(a.loc);
     const T* attn = static_cast<const T*>(a.attn);
     T* out = static_cast<T*>(a.out);
     const __amdgpu_buffer_rsrc_t vres =
@@ -146,8 +145,8 @@ __global__ __launch_bounds__(LDSC ? 512 : 256) void msda_fwd_kernel(const KArgs 
         r.x = 0.f, r.y = 0.f, r.aw = 0.f, r.l = 0;
         if (r.active) {
             const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
-            r.x = to_f32(loc[2 * sr.loc_e]);
-            r.y = to_f32(loc[2 * sr.loc_e + 1]);
+            r.x = load_coord<SRC, T>(a.loc, 2 * sr.loc_e);
+            r.y = load_coord<SRC, T>(a.loc, 2 * sr.loc_e + 1);
             if constexpr (SRC == kSrcGrid) r.aw = 1.0f;  // no weights tensor
             else r.aw = to_f32(attn[sr.w_e]);
             r.l = sr.l;

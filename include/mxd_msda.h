@@ -242,7 +242,9 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
 /* ---- geometric kernel attention --------------------------------------------------------------
  * Replaces geometric_kernel_attention_forward / _backward (mx_driving/csrc/GeometricKernelAttentionFunc.cpp:33-118)
  * with the operator's own layouts: value [bs, nk, nh, hd] (the reference's binding permutes it itself),
- * sampling_locations [bs, nq, nh, nl, np, 2] = (x, y) pixel indices in value's dtype (clamped to the level),
+ * sampling_locations [bs, nq, nh, nl, np, 2] = (x, y) pixel indices as FLOAT32 whatever `dtype` is (the reference takes
+ * float16/float32/int32/int64 locations, GeometricKernelAttentionFunc.cpp:40-44; a 16-bit float cannot hold the indices
+ * of a level wider than 2048 pixels, so a binding converts to float32, which is exact below 2^24), clamped to the level,
  * attn_weights [bs, nq, nh, nl, np], output [bs, nq, nh*hd]:
  *   output[b,q,h,:] = sum over (l, p) of attn * value[b, start_l + y*W_l + x, h, :].
  * Gradients: grad_value and grad_attn_weights (locations are indices and have none). */

@@ -81,3 +81,39 @@ def test_random_small_problems(gpu_device, seed):
     got = run_gpu(*inp, gpu_device)
     for g_, w_, tol in zip(got, want, (FWD_FP32, BWD_FP32, BWD_FP32)):
         assert rel_err(g_, w_) <= tol
+
+
+@pytest.mark.parametrize("dtype,loc_dtype,hw", [(torch.bfloat16, torch.float32, (3, 700)), (torch.float16, torch.float32, (2, 3000)),
+                                                (torch.float16, torch.int64, (2, 3000)), (torch.bfloat16, torch.int32, (700, 3)),
+                                                (torch.float16, torch.float16, (5, 40))])
+def test_levels_wider_than_a_16bit_float_can_index(gpu_device, dtype, loc_dtype, hw):
+    """Pixel indices beyond 256 (bfloat16) / 2048 (float16) are not representable in value's 16-bit dtype; locations
+    travel to the kernels as float32 whatever value's dtype is (the reference accepts float16 values with
+    float32 / int32 / int64 locations, mx_driving/csrc/GeometricKernelAttentionFunc.cpp:40-44)."""
+    bs, nq, hd, nh, nl, npts = 2, 300, 16, 2, 1, 5
+    g = torch.Generator().manual_seed(hw[1])
+    sh = torch.tensor([list(hw)])
+    lsi = torch.zeros(1, dtype=torch.int64)
+    loc = torch.stack((torch.randint(-2, hw[1] + 2, (bs, nq, nh, nl, npts), generator=g),
+                       torch.randint(-2, hw[0] + 2, (bs, nq, nh, nl, npts), generator=g)), -1).float()
+    loc[0, 0, 0, 0, 0] = torch.tensor([hw[1] - 1.0, hw[0] - 1.0])   # the last pixel itself
+    value = torch.rand(bs, hw[0] * hw[1], nh, hd, generator=g) * 3
+    attn = torch.rand(bs, nq, nh, nl, npts, generator=g)
+    go = torch.rand(bs, nq, nh * hd, generator=g)
+    v16, a16, g16 = value.to(dtype).double(), attn.to(dtype).double(), go.to(dtype).double()
+    loc_in = loc.to(loc_dtype)
+    want = (gka.forward(v16, sh, lsi, loc_in.double(), a16),) + gka.backward(v16, sh, lsi, loc_in.double(), a16, g16)
+    got = run_gpu(value, sh, lsi, loc_in, attn, go, gpu_device, dtype=dtype, loc_dtype=loc_dtype)
+    tol = HALF if dtype == torch.float16 else 2.0 ** -8
+    for name, g_, w_ in zip(("output", "grad_value", "grad_attn_weights"), got, want):
+        assert rel_err(g_, w_) <= tol, (name, rel_err(g_, w_))
+
+
+def test_largest_reference_shape_at_full_batch(gpu_device):
+    """The largest shape of the reference's test at its full batch size, [24, 7156, 64, 4, 1, 15]
+    (tests/torch/test_geometric_kernel_attention.py:112-119) -- the shape bench.py times."""
+    inp = make_inputs([24, 7156, 64, 4, 1, 15], (15, 25), seed=7156)
+    want = (gka.forward(*inp[:5]),) + gka.backward(*inp)
+    got = run_gpu(*inp, gpu_device)
+    for name, g_, w_, tol in zip(("output", "grad_value", "grad_attn_weights"), got, want, (FWD_FP32, BWD_FP32, BWD_FP32)):
+        assert rel_err(g_, w_) <= tol, (name, rel_err(g_, w_))

@@ -114,3 +114,11 @@ def test_channels_last_input_keeps_its_memory_format(gpu_device):
     xr = x.double().requires_grad_()
     F.grid_sample(xr, grid.double(), "bilinear", "zeros", False).backward(go.double())
     assert rel_err(xcl.grad.double().cpu().numpy(), xr.grad.numpy()) <= BWD_FP32
+
+
+def test_largest_reference_shape_at_full_batch(gpu_device):
+    """The largest shape of the reference's test at its full batch size, input [24, 128, 64, 176], grid [24, 24, 176, 2]
+    (tests/torch/test_grid_sampler2d_v2.py:34-59) -- the shape bench.py times (float64 grid_sample on the CPU takes a few
+    seconds at this size)."""
+    x, grid, go = make_inputs([24, 128, 64, 176], [24, 24, 176, 2], seed=24)
+    print(check(x, grid, go, "zeros", False, gpu_device))

@@ -216,3 +216,110 @@ def test_fused_backward_workspace_adds_the_reference_point_partials():
     assert lib.mxd_msda_fused_backward_workspace_bytes(*args, 2, 1) == plain + 8 * 2 * 19947 * 4 * 2 * 4
     assert lib.mxd_msda_fused_backward_workspace_bytes(*args, 4, 1) == plain + 8 * 2 * 19947 * 4 * 4 * 4
     assert lib.mxd_msda_fused_backward_workspace_bytes(*args, 3, 1) == 0
+
+
+def test_reference_module_paths_below_the_package_root():
+    """The reference's operator files do ``import mx_driving._C`` (mx_driving/ops/multi_scale_deformable_attn.py:15,38)
+    and its package re-exports from ``.ops.<operator>`` (mx_driving/__init__.py:106-113): both paths resolve, to the
+    same objects, and ``_C`` carries the names the reference binds (mx_driving/csrc/pybind.cpp:110-111,121-122,131-132,
+    205-208)."""
+    import importlib
+    c = importlib.import_module("mx_driving._C")
+    for name in ("multi_scale_deformable_attn", "multi_scale_deformable_attn_backward", "npu_deformable_aggregation",
+                 "npu_deformable_aggregation_backward", "geometric_kernel_attention_forward",
+                 "geometric_kernel_attention_backward", "grid_sampler2d_v2", "grid_sampler2d_v2_backward"):
+        assert callable(getattr(c, name)), name
+    assert c.multi_scale_deformable_attn is _C.multi_scale_deformable_attn
+    assert c.npu_deformable_aggregation is _C.deformable_aggregation
+    m = importlib.import_module("mx_driving.ops.multi_scale_deformable_attn")
+    assert m.MultiScaleDeformableAttnFunction is mx_driving.MultiScaleDeformableAttnFunction
+    assert m.multi_scale_deformable_attn is mx_driving.multi_scale_deformable_attn
+    assert importlib.import_module("mx_driving.ops.npu_deformable_aggregation").npu_deformable_aggregation \
+        is mx_driving.npu_deformable_aggregation
+    assert importlib.import_module("mx_driving.ops.geometric_kernel_attention").geometric_kernel_attention \
+        is mx_driving.geometric_kernel_attention
+    assert importlib.import_module("mx_driving.ops.grid_sampler2d_v2").grid_sampler2d_v2 is mx_driving.grid_sampler2d_v2
+
+
+C_PROGRAM = r"""
+/* A C99 host: the header compiles as C, the library links, and the entry points that need no GPU behave. */
+#include <stdio.h>
+#include <string.h>
+#include "mxd_msda.h"
+
+int main(void)
+{
+    mxd_msda_plan plan;
+    int32_t work[4];
+    int rc;
+    if (mxd_msda_version() != MXD_MSDA_VERSION) return 1;
+    if (strcmp(mxd_msda_last_error(), "") != 0) return 2;
+    rc = mxd_msda_make_plan(0, MXD_DTYPE_F32, 2, 19947, 8, 32, 4, 4, 19947, 4, 16, &plan);
+    if (rc != MXD_OK || plan.vec != 4 || plan.lanes_per_row != 8 || plan.grid == 0) return 3;
+    if (!mxd_msda_decode_block(&plan, 0, 2, 8, 19947, work) || work[0] != 0 || work[2] != 0) return 4;
+    if (mxd_msda_make_plan(0, 7, 1, 10, 1, 32, 1, 1, 1, 1, 16, &plan) != MXD_E_DTYPE) return 5;
+    if (mxd_msda_make_plan(0, MXD_DTYPE_F16, 1, 10, 1, 257, 1, 1, 1, 1, 16, &plan) != MXD_E_SHAPE) return 6;
+    if (strstr(mxd_msda_last_error(), "256") == NULL) return 7;
+    if (mxd_msda_make_plan(0, MXD_DTYPE_F32, 1, 10, 1, 32, 1, 1, 1, 1, 16, NULL) != MXD_E_NULL) return 8;
+    if (mxd_msda_forward(NULL, NULL, NULL, NULL, NULL, NULL, MXD_DTYPE_F32, 1, 10, 1, 32, 1, 1, 1, 1, NULL) != MXD_E_NULL)
+        return 9;
+    if (mxd_msda_backward_workspace_bytes(MXD_DTYPE_F32 | MXD_META_I64, 2, 100, 8, 32, 4, 4, 50, 3) == 0) return 10;
+    if (mxd_msda_backward_workspace_bytes(MXD_DTYPE_F32, 2, 100, 8, 300, 4, 4, 50, 3) != 0) return 11;
+    if (mxd_msda_backward_static_limit() != MXD_MSDA_STATIC_SCRATCH_BYTES) return 12;
+    printf("ok %d\n", mxd_msda_version());
+    return 0;
+}
+"""
+
+
+def test_header_compiles_as_c99_and_the_library_links(tmp_path):
+    """include/mxd_msda.h through a C compiler (not C++), linked against the built library, run."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "host.c"
+    src.write_text(C_PROGRAM)
+    exe = tmp_path / "host"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"),
+                    str(src), "-o", str(exe), "-L", libdir, "-lmxd_msda", f"-Wl,-rpath,{libdir}",
+                    "-Wl,-rpath,/opt/rocm/lib"], check=True, capture_output=True, text=True)
+    res = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert res.returncode == 0, (res.returncode, res.stdout, res.stderr)
+    assert res.stdout.startswith("ok 100")
+
+
+def test_backward_runs_every_fallible_step_before_its_first_launch(monkeypatch):
+    """A problem that passes the size checks and the workspace check but whose grad_value pass would need more
+    workgroups than a launch can have: the call must fail with MXD_E_SHAPE having enqueued nothing.  Without a GPU a
+    launch attempted first would have surfaced as MXD_E_LAUNCH instead.  (No pointer is dereferenced on the host.)"""
+    if torch.cuda.is_available():
+        pytest.skip("meant for a box without a GPU: the sizes describe terabytes of (never touched) memory")
+    from util import set_tuning
+    set_tuning(monkeypatch, MXD_MSDA_TILE_TARGET=128)   # (small work items: 259 per (batch, head) here)
+    lib = _lib.load()
+    dims = (1 << 20, 64, 8, 32, 1, 1, 32, 512)   # bs, nk, nh, hd, nl, nl_attn, nq, np
+    need = lib.mxd_msda_backward_workspace_bytes(0, *dims)
+    assert need > 0
+    fake = 4096   # a non-NULL, 16-byte aligned value standing for device pointers that are never used
+    rc = lib.mxd_msda_backward(fake, fake, fake, fake, fake, fake, fake, fake, fake, fake, need, 0, *dims, 0, None)
+    assert rc == -2, (rc, _lib.last_error())
+    assert "workgroups" in _lib.last_error()
+
+
+def test_backward_plans_stay_inside_the_default_lds_limit():
+    """The first backward kernel does not opt in to more than 64 KiB of LDS: for every row size and up to the largest
+    key count a call accepts its plan must fit, the launcher falling back to the one-kernel form (no tile counters in
+    LDS) where the tile bookkeeping would not."""
+    for dtype in (0, 1, 2):
+        for hd in (1, 4, 8, 16, 32, 64, 128, 256):
+            es = 4 if dtype == 0 else 2
+            for nh in (1, 8):
+                limit = ((1 << 31) - 1) // (nh * hd * 4)
+                for nk in (1000, 500_000, 1_800_000, 2_090_000, 16_000_000, limit):
+                    if nk > limit:
+                        continue
+                    for nl in (1, 4):
+                        plan = _lib.make_plan(1, dtype, 1, nk, nh, hd, nl, nl, 1000, 4)
+                        assert plan.lds_bytes <= 64 * 1024, (dtype, hd, nh, nk, nl, plan.lds_bytes, es)

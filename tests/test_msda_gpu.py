@@ -10,7 +10,8 @@ import torch
 
 from drivingsdk_amd import _lib, workloads
 from oracle import msda_oracle as orc
-from util import BWD_FP32, FWD_FP32, HALF, oracle_all, rel_err, run_gpu, set_tuning, to_device
+from util import (BF16, BWD_FP32, FWD_FP32, HALF, check_16bit, check_close, half_tol, level_slices, oracle_all, rel_err,
+                  run_gpu, set_tuning, to_device)
 
 pytestmark = pytest.mark.gpu
 
@@ -35,21 +36,39 @@ def _cell_edge_mask(inp):
 
 
 def _check_all(inp, device, fwd_tol, bwd_tol, with_grads=True):
+    """HIP path against the float64 oracle on the same inputs: the max-norm figure the path's tolerances are stated in,
+    and element-wise -- float32: |got - ref| <= tol * (|ref| + RMS of the element's level); 16-bit: within one unit in
+    the last place of the oracle rounded to the storage type.  grad_value and the per-sample gradients are also held
+    to the max-norm tolerance level by level (the coarse level collects a quarter of the samples in a few hundred rows
+    and would otherwise set the scale for all of them)."""
     ref = oracle_all(inp, with_grads)
     got = run_gpu(inp, device, with_grads)
+    dtype = inp.value.dtype
     errs = {}
     names = ("output", "grad_value", "grad_sampling_locations", "grad_attention_weights")
     for name, g, r, tol in zip(names, got, ref, (fwd_tol, bwd_tol, bwd_tol, bwd_tol)):
         if r is None:
             continue
+        r = np.asarray(r)
         if name == "grad_sampling_locations":
             edge = _cell_edge_mask(inp)
-            assert edge.mean() < 1e-4, "too many samples sit on a cell edge for this check to mean anything"
+            assert edge.mean() < 1e-4 or dtype != torch.float32, "too many samples sit on a cell edge for this check to mean anything"
             keep = ~edge[..., None]
             g, r = g * keep, r * keep
             errs["cell_edge_samples"] = int(edge.sum())
         errs[name] = rel_err(g, r)
         assert errs[name] <= tol, (name, errs)
+        groups = None if name == "output" else level_slices(inp, "keys" if name == "grad_value" else "samples")
+        nl = inp.spatial_shapes.shape[0]
+        if groups is not None and name != "grad_value":
+            groups = groups[:nl]   # (extra level slots of the weights carry zeros)
+        for idx in (groups or []):
+            if np.abs(r[idx]).max() > 0:
+                assert rel_err(g[idx], r[idx]) <= tol, (name, "level", idx, rel_err(g[idx], r[idx]))
+        if dtype == torch.float32:
+            check_close(g, r, tol, name, groups)
+        else:
+            check_16bit(g, r, dtype, name, groups, tol32=FWD_FP32 if name == "output" else BWD_FP32)
     return errs
 
 
@@ -102,8 +121,7 @@ def test_bevformer_sca_forward(gpu_device, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_head_dim_128_forward_and_backward(gpu_device, dtype):
     inp = workloads.make_inputs("head_dim_128", dtype=dtype, with_grad_output=True)
-    # bfloat16 carries 8 mantissa bits: one rounding of the result is 2^-9 = 1.95e-3 relative
-    tol = HALF if dtype == torch.float16 else 4e-3
+    tol = half_tol(dtype)   # (bfloat16: its unit round-off, 2^-8)
     errs = _check_all(inp, gpu_device, tol, tol)
     print("head_dim_128", dtype, errs)
 
@@ -207,8 +225,7 @@ def test_odd_head_dims_and_head_counts(gpu_device, hd, nh, dtype):
     gout = torch.randn(bs, nq, nh * hd, generator=g)
     inp = workloads.MsdaInputs(*[t.to(dtype) if t.is_floating_point() else t for t in
                                  (value, shapes, lsi, loc, attn, gout)])
-    tol_f, tol_b = (FWD_FP32, BWD_FP32) if dtype == torch.float32 else \
-        ((HALF, HALF) if dtype == torch.float16 else (4e-3, 4e-3))
+    tol_f, tol_b = (FWD_FP32, BWD_FP32) if dtype == torch.float32 else (half_tol(dtype), half_tol(dtype))
     errs = _check_all(inp, gpu_device, tol_f, tol_b)
     print(hd, nh, dtype, errs)
 
@@ -487,7 +504,7 @@ def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
     """The forward's level cache (rows of the last levels held in LDS) is switched by an estimate of the level
     sizes; here it is forced off and on with room for no, one, several and all levels, for every dtype."""
     set_tuning(monkeypatch, MXD_MSDA_FWD_LDS=lds, MXD_MSDA_FWD_CU=0)   # (the general forward kernel's cache)
-    tol = FWD_FP32 if dtype == torch.float32 else (HALF if dtype == torch.float16 else 2.0 ** -8)
+    tol = FWD_FP32 if dtype == torch.float32 else half_tol(dtype)
     for name, scale in (("tiny", 1.0), ("detr_encoder", 0.1)):
         inp = workloads.make_inputs(name, dtype=dtype, scale_queries=scale)
         want = oracle_all(inp, with_grads=False)[0]
@@ -660,7 +677,7 @@ def test_random_small_problems_16bit(gpu_device, seed):
                                inp.sampling_locations.to(dtype), inp.attention_weights.to(dtype),
                                inp.grad_output.to(dtype))
     print("case", desc, dtype, flush=True)
-    tol = HALF if dtype == torch.float16 else 2.0 ** -8
+    tol = half_tol(dtype)
     ref = oracle_all(inp)
     got = run_gpu(inp, gpu_device)
     # 16-bit locations sit on cell edges far more often than float32 ones: the location gradient is compared away
@@ -725,9 +742,27 @@ def test_random_small_problems_cu_form(gpu_device, monkeypatch, seed):
     print("case", (bs, nq, nh, hd, levels, npts), dtype, flush=True)
     want = oracle_all(inp, with_grads=False)[0]
     got = run_gpu(inp, gpu_device, with_grads=False)[0]
-    tol = FWD_FP32 if dtype == torch.float32 else (HALF if dtype == torch.float16 else 2.0 ** -8)
+    tol = FWD_FP32 if dtype == torch.float32 else half_tol(dtype)
     assert rel_err(got, want) <= tol
     with monkeypatch.context() as m:
         set_tuning(m, MXD_MSDA_FWD_CU=0)
         general = run_gpu(inp, gpu_device, with_grads=False)[0]
     assert np.array_equal(np.asarray(got), np.asarray(general))
+
+
+def test_backward_with_more_tiles_than_the_lds_bookkeeping_holds(gpu_device):
+    """One level of 2.09 M pixels and 64-byte rows (a 1080x1920 grid-sampler-like input): the per-tile counters of the
+    first backward kernel would not fit the LDS next to 16 units' staging strips, so the launcher takes the
+    one-kernel form with global atomics.  Gradients against the oracle."""
+    g = torch.Generator().manual_seed(2090)
+    levels = ((1100, 1900),)
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = 1100 * 1900
+    bs, nq, nh, hd, npts = 1, 2000, 1, 16, 4
+    plan = _lib.make_plan(1, 0, bs, nk, nh, hd, 1, 1, nq, npts)
+    assert plan.lds_bytes <= 64 * 1024 and plan.iters == 1      # (the atomic form: one iteration per wavefront)
+    assert _lib.load().mxd_msda_backward_workspace_bytes(0, bs, nk, nh, hd, 1, 1, nq, npts) == 0
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g), shapes, lsi,
+                               torch.rand(bs, nq, nh, 1, npts, 2, generator=g) * 1.02 - 0.01,
+                               torch.rand(bs, nq, nh, 1, npts, generator=g), torch.randn(bs, nq, nh * hd, generator=g))
+    print(_check_all(inp, gpu_device, FWD_FP32, BWD_FP32))
