@@ -387,7 +387,22 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
     const int cap = mxd::kCuLdsBytes - mxd::kCuTableBytes;  // (two level tables come first)
     const int64_t cap_rows = cap / (d.hd * es) - 1;
     const int64_t cached = estimated_cached_rows(d, cap_rows);
-    if (mode < 0 && (cached == 0 || d.bs * d.nh * d.nq * d.nl * d.np < (int64_t(1) << 20))) return false;
+    // By default (measured on MI355X): the form wins where about half of the samples are gathered from LDS and a unit's
+    // samples are one chunk -- the Deformable-DETR encoder shape, 84 against 97 us in float32 and 72 against 88 us in
+    // float16 -- and does not where a quarter are or a unit takes two chunks (BEVFormer's eight points per level:
+    // float32 389 against 420 us, float16 346 against 278 us; head_dim 128: equal), where the general kernel stays.
+    if (mode < 0) {
+        double last = (double)d.nk, rows = 0.0;
+        if (d.nl > 1) last = (double)d.nk * 3.0 / ((double)(int64_t(1) << (2 * (d.nl < 16 ? d.nl : 16))) - 1.0);
+        int levels_cached = 0;
+        for (double r = last; levels_cached < d.nl && rows + r <= (double)cap_rows; r *= 4.0) {
+            rows += r;
+            ++levels_cached;
+        }
+        if (2 * levels_cached < d.nl || d.nl * d.np > mxd::kChunk ||
+            d.bs * d.nh * d.nq * d.nl * d.np < (int64_t(1) << 20))
+            return false;
+    }
     const int U = mxd::kWave / lpr;
     const int64_t groups = (d.nq + U - 1) / U;
     // Workgroups per (batch, head): every XCD has 32 CUs, each of which runs one workgroup at a time; the launch
@@ -398,6 +413,7 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
     double best_cost = -1.0;
     const int64_t max_p = groups < 512 ? groups : 512;
     const double slice_bytes = (double)(d.nk - cached) * (double)(d.hd * es);
+    const double launch = 3000.0, fill = (double)cached + 1000.0;   // in units of one gathered row
     for (int64_t P = 1; P <= max_p; ++P) {
         if (tuning().fwd_cu_wgs > 0 && P != tuning().fwd_cu_wgs && tuning().fwd_cu_wgs <= max_p) continue;
         const int64_t tq = U * (((d.nq + P - 1) / P + U - 1) / U);
@@ -411,9 +427,12 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
         if (trial.xcd_mode == 1 && slices < (double)trial.heads_per_xcd) slices = (double)trial.heads_per_xcd;
         if (trial.xcd_mode == 0) slices = slices * 8.0 < (double)d.nh ? (double)d.nh : slices * 8.0;
         if (slices < 1.0) slices = 1.0;
-        double over = ceil(slices) * slice_bytes / (4.0 * 1024 * 1024) - 0.8;
+        // (measured at the encoder shape: two slices side by side cost 10 to 15 % also where both fit the L2 --
+        //  float16, 2 x 1.2 MB -- and 15 to 25 % where they do not -- float32, 2 x 2.4 MB)
+        double over = ceil(slices) * slice_bytes / (4.0 * 1024 * 1024) - 0.4;
         over = over < 0.0 ? 0.0 : (over > 1.0 ? 1.0 : over);
-        const double cost = rounds * ((double)cached + 3000.0 + (1.0 + 0.5 * over) * (double)tq * (double)(d.nl * d.np) * 4.0);
+        const double gather = (1.0 + 0.5 * over) * (double)tq * (double)(d.nl * d.np) * 4.0;
+        const double cost = rounds * (launch + fill + gather);
         if (best_cost < 0.0 || cost < best_cost) {
             best_cost = cost;
             best_p = P;

@@ -74,7 +74,7 @@ def _check_all(inp, device, fwd_tol, bwd_tol, with_grads=True):
 
 def test_library_is_the_in_tree_build():
     lib = _lib.load()
-    assert lib.mxd_msda_version() == 100
+    assert lib.mxd_msda_version() == 101
     with open("/proc/self/maps") as f:
         assert any("drivingsdk_amd/lib/libmxd_msda.so" in line for line in f)
 
@@ -700,19 +700,23 @@ def test_random_small_problems_16bit(gpu_device, seed):
                                         ("bevformer_sca", torch.float16), ("head_dim_128", torch.float16),
                                         ("head_dim_128", torch.bfloat16)])
 def test_forward_cu_form_equals_the_general_form_at_full_size(gpu_device, monkeypatch, name, dtype):
-    """The benchmark shapes take the forward's one-workgroup-per-CU form by default (last levels in LDS, sample values
-    handed across lanes by DPP; rows of 8, 4 and 16 lanes here).  Its sums run in the same order as the general
-    kernel's, so at full size the two must agree bit for bit; the general kernel is checked against the oracle at these
-    sizes elsewhere."""
+    """The forward's one-workgroup-per-CU form (last levels in LDS, sample values handed across lanes by DPP; rows of 8,
+    4 and 16 lanes here) at the benchmark shapes: the encoder shape takes it by default, the others are made to.  Its
+    sums run in the same order as the general kernel's, so at full size the two must agree bit for bit; the general
+    kernel is checked against the oracle at these sizes elsewhere."""
     from drivingsdk_amd import _C
     d = to_device(workloads.make_inputs(name, dtype=dtype), gpu_device)
     args = (d.value, d.spatial_shapes, d.level_start_index, d.sampling_locations, d.attention_weights)
-    plan = _lib.make_plan(0, {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype], *d.value.shape,
-                          d.spatial_shapes.shape[0], d.spatial_shapes.shape[0], d.sampling_locations.shape[1],
-                          d.sampling_locations.shape[4])
-    assert plan.block == 1024, "the benchmark shapes are meant to take the one-workgroup-per-CU form"
+    dims = (*d.value.shape, d.spatial_shapes.shape[0], d.spatial_shapes.shape[0], d.sampling_locations.shape[1],
+            d.sampling_locations.shape[4])
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    if name == "detr_encoder":
+        assert _lib.make_plan(0, code, *dims).block == 1024, "the encoder shape is meant to take this form by default"
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=1)
+    assert _lib.make_plan(0, code, *dims).block == 1024
     out_cu = _C.multi_scale_deformable_attn(*args)
     set_tuning(monkeypatch, MXD_MSDA_FWD_CU=0)
+    assert _lib.make_plan(0, code, *dims).block != 1024
     out_general = _C.multi_scale_deformable_attn(*args)
     assert torch.equal(out_cu, out_general)
 
