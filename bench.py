@@ -90,7 +90,9 @@ def _kernel_times(d, iters, warmup):
                                    ws.data_ptr(), ws_bytes, code, *dims, flags, stream)
         assert rc == 0, _lib.last_error()
 
-    res = {"forward_ms": _event_ms(fwd, iters, warmup), "backward_with_zero_fill_ms": _event_ms(lambda: bwd(0), iters, warmup)}
+    plan = _lib.make_plan(0, code, *dims)
+    res = {"forward_kernel": "msda_fwd_cu_kernel" if plan.block == 1024 else "msda_fwd_kernel",
+           "forward_ms": _event_ms(fwd, iters, warmup), "backward_with_zero_fill_ms": _event_ms(lambda: bwd(0), iters, warmup)}
     n_single = min(max(iters, 20), 100)
     res["forward_single_launch_ms"] = _event_stats_ms(fwd, n_single)
     res["backward_single_launch_ms"] = _event_stats_ms(lambda: bwd(0), n_single)
@@ -166,33 +168,77 @@ def _committed_traffic(workload, dtype):
     return data["kernels"]
 
 
-def _cpu_baseline(inp, max_seconds=25.0):
-    """The CPU oracle (grid_sample formulation, float32, autograd backward) on the host cores:
-    whole forward+backward iterations of the same workload, as many as fit the time bound."""
+def _physical_cores():
+    """Physical cores of the host (psutil when importable, else distinct (package, core) pairs of /proc/cpuinfo)."""
+    try:
+        import psutil
+        n = psutil.cpu_count(logical=False)
+        if n:
+            return int(n)
+    except Exception:
+        pass
+    try:
+        pairs, pkg = set(), None
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("physical id"):
+                    pkg = line.split(":")[1].strip()
+                elif line.startswith("core id"):
+                    pairs.add((pkg, line.split(":")[1].strip()))
+        return len(pairs) or None
+    except OSError:
+        return None
+
+
+def _cpu_baseline(inp, max_seconds=16.0):
+    """The CPU oracle (grid_sample formulation, float32, autograd backward) on the host cores: whole forward+backward
+    iterations of the same workload, as many as fit the time bound -- with the threads this process may use (torch's
+    default: the box's CPU share) and, for reference, with one thread."""
     import torch
 
     from oracle import msda_oracle as orc
 
+    def run(threads, bound, most):
+        torch.set_num_threads(threads)
+        times = []
+        t_begin = time.perf_counter()
+        it = 0
+        while True:
+            t0 = time.perf_counter()
+            orc.msda_grid_sample_fwd_bwd(inp.value, inp.spatial_shapes, inp.sampling_locations, inp.attention_weights,
+                                         inp.grad_output, dtype=torch.float32)
+            t1 = time.perf_counter()
+            if it > 0:  # first iteration is a warm-up
+                times.append(t1 - t0)
+            it += 1
+            if len(times) >= most or ((time.perf_counter() - t_begin) > bound and times):
+                break
+        return statistics.median(times), len(times)
+
     threads = torch.get_num_threads()
-    times = []
-    t_begin = time.perf_counter()
-    it = 0
-    while True:
-        t0 = time.perf_counter()
-        orc.msda_grid_sample_fwd_bwd(inp.value, inp.spatial_shapes, inp.sampling_locations, inp.attention_weights,
-                                     inp.grad_output, dtype=torch.float32)
-        t1 = time.perf_counter()
-        if it > 0:  # first iteration is a warm-up
-            times.append(t1 - t0)
-        it += 1
-        if len(times) >= 5 or (time.perf_counter() - t_begin) > max_seconds and times:
-            break
-    med = statistics.median(times)
     nqueries = inp.sampling_locations.shape[0] * inp.sampling_locations.shape[1]
+    med, n = run(threads, max_seconds, 5)
+    med1, n1 = run(1, max_seconds, 2)
+    torch.set_num_threads(threads)
     return {"value": nqueries / med, "unit": "queries/s", "cores": threads, "kind": "port",
-            "ms_per_step": med * 1e3,
-            "sample": f"{len(times)} timed forward+backward iterations (median) of the full workload after 1 warm-up, "
-                      f"torch grid_sample formulation in float32 with {threads} threads"}
+            "ms_per_step": med * 1e3, "host_physical_cores": _physical_cores(), "host_logical_cpus": os.cpu_count(),
+            "single_thread": {"value": nqueries / med1, "unit": "queries/s", "cores": 1, "ms_per_step": med1 * 1e3,
+                              "sample": f"{n1} timed iteration(s) after 1 warm-up"},
+            "sample": f"{n} timed forward+backward iterations (median) of the full workload after 1 warm-up, "
+                      f"torch grid_sample formulation in float32 with {threads} threads (the CPU share of a one-GPU box)"}
+
+
+def _copy_bandwidth_gbps():
+    """Measured device copy bandwidth (bytes read + bytes written per second) of a 1 GiB device-to-device copy: the
+    figure to hold next to the published 8 TB/s."""
+    import torch
+
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    src.zero_()
+    ms = _event_ms(lambda: dst.copy_(src), iters=10, warmup=3)
+    return 2.0 * n / (ms * 1e-3) / 1e9
 
 
 def _bench_dagg(args):
@@ -440,6 +486,7 @@ def main():
     k = _kernel_times(d, iters=max(args.steps, 50), warmup=max(args.warmup, 10))
 
     traffic = _committed_traffic(args.workload, args.dtype)
+    copy_gbps = _copy_bandwidth_gbps()
 
     def roof(nbytes, ms, kernels):
         achieved = nbytes / (ms * 1e-3) / 1e9
@@ -448,9 +495,9 @@ def main():
             hbm = sum(traffic[k]["hbm_bytes"] for k in kernels)
         return {"bound": "hbm", "kernel": " + ".join(kernels), "achieved": achieved, "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": hbm, "algorithmic_bytes": nbytes,
-                "kernel_ms": ms}
+                "kernel_ms": ms, "measured_copy_GBps": copy_gbps, "frac_of_measured_copy": achieved / copy_gbps}
 
-    roof_fwd = roof(bytes_fwd, k["forward_ms"], ["msda_fwd_kernel"])
+    roof_fwd = roof(bytes_fwd, k["forward_ms"], [k["forward_kernel"]])
     # the backward pass: per-sample dots (grad_attn, grad_loc, records; its workgroups also zero-fill the image),
     # then grad_value by tile ownership
     roof_bwd = roof(bytes_bwd, k["backward_with_zero_fill_ms"], ["msda_bwd_kernel", "msda_gradv_tiles_kernel"])

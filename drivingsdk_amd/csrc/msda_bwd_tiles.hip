@@ -137,7 +137,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
 
     Work wk;
     if (!decode_block(t.map, blockIdx.x, a.bs, a.nh, t.items_per_bh, &wk)) return;
-    {
+    if (t.batch_major == 0) {
         // item-major, batch-minor: the long-running items (coarse levels, numbered first) of every
         // batch element start at the beginning of the launch
         const int64_t r = (int64_t)wk.b * t.items_per_bh + wk.q_begin;

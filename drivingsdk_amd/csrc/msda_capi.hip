@@ -78,6 +78,7 @@ struct Tuning {
                          // -1 = for problems large enough to pay for it
     int fwd_cu_wgs;      // MXD_MSDA_FWD_CU_WGS: its workgroups per (batch, head), 0 = chosen here
     int bwd_fill_kernel; // MXD_MSDA_BWD_FILL_KERNEL: 1 = zero-fill by a kernel of its own
+    int tile_order;      // MXD_MSDA_TILE_ORDER: 1 = work items of the tile pass batch-major, 0 = item-major, -1 = chosen here
 };
 Tuning g_tuning;
 std::once_flag g_tuning_once;
@@ -96,6 +97,7 @@ void read_tuning()
     t.fwd_cu = env_int("MXD_MSDA_FWD_CU", -1);
     t.fwd_cu_wgs = env_int("MXD_MSDA_FWD_CU_WGS", 0);
     t.bwd_fill_kernel = env_int("MXD_MSDA_BWD_FILL_KERNEL", 0);
+    t.tile_order = env_int("MXD_MSDA_TILE_ORDER", -1);
     g_tuning = t;
 }
 
@@ -332,6 +334,7 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
     t->items_per_bh = (int32_t)items;
     t->vec = vec;
     t->accumulate = accumulate;
+    t->batch_major = tuning().tile_order > 0 ? 1 : 0;
     t->map.tile_q = 1;
     const int64_t grid = fill_xcd_map(&t->map, d.bs, d.nh, items);
     if (grid >= (int64_t(1) << 31)) return fail(MXD_E_SHAPE, "backward needs %lld workgroups, beyond the launch limit", (long long)grid);

@@ -119,6 +119,8 @@ struct TileArgs {
     int32_t vec;           // elements per load of a grad_out row
     int32_t accumulate;    // add into the existing contents of the image
     int32_t store_vec;     // 4: rows of the image are 16-byte aligned, else 1
+    int32_t batch_major;   // 1: the work items of a batch element are numbered together (an XCD's L2 then holds one
+                           // batch element's grad_out rows at a time); 0: item-major across batch elements
     uint32_t grid, block;
 };
 
