@@ -48,7 +48,22 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     if constexpr (!SCATTER) {
         // this workgroup's share of the zero-fill of the image (every workgroup of the launch takes one, also those
         // without work): the stores ride along with this kernel instead of taking a launch of their own
-        if (a.fill_n4 != 0) {
+        if (a.fill_n4 != 0 && a.sparse != 0) {
+            // only the rows that receive atomic additions in the tile pass (tiles split by query range, small tiles,
+            // and the first pixel of every other tile); a row of the image is nh*hd floats, a multiple of 16 bytes here
+            const int32_t tiles = a.tbl_stride - 1;  // (bound: pieces of tiles that do not exist are skipped)
+            const int64_t pieces = (int64_t)a.bs * tiles * kRowParts;
+            const uint32_t row4 = (uint32_t)(a.nh * a.hd) / 4;
+            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            for (int64_t w = blockIdx.x; w < pieces; w += gridDim.x) {
+                const int32_t b = (int32_t)(w / (tiles * kRowParts)), r = (int32_t)(w % (tiles * kRowParts));
+                int32_t r0, r1;
+                if (!atomic_rows_of_part(a, r / kRowParts, r % kRowParts, &r0, &r1)) continue;
+                f32x4* img = reinterpret_cast<f32x4*>(a.grad_value) + ((size_t)b * a.nk + r0) * row4;
+                const uint32_t n4 = (uint32_t)(r1 - r0) * row4;
+                for (uint32_t i = threadIdx.x; i < n4; i += blockDim.x) __builtin_nontemporal_store(z, img + i);
+            }
+        } else if (a.fill_n4 != 0) {
             f32x4* img = reinterpret_cast<f32x4*>(a.grad_value);
             const uint64_t per = (a.fill_n4 + gridDim.x - 1) / gridDim.x;
             const uint64_t lo = (uint64_t)blockIdx.x * per;
@@ -662,6 +677,39 @@ __global__ __launch_bounds__(256) void msda_round_kernel(const float* src, T* ds
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) dst[i] = from_f32<T>(src[i]);
+}
+
+// 16-bit dtypes, sparse image: rounds the rows of the fp32 image that received atomic additions into the caller's
+// tensor (the other rows were stored there by the tile pass).  One workgroup per piece of a tile of a batch element.
+template <typename T>
+__global__ __launch_bounds__(256) void msda_round_rows_kernel(const KArgs a)
+{
+    const int32_t tiles = a.tbl_stride - 1;
+    const int32_t b = (int32_t)(blockIdx.x / (uint32_t)(tiles * kRowParts)), r = (int32_t)(blockIdx.x % (uint32_t)(tiles * kRowParts));
+    int32_t r0, r1;
+    if (b >= a.bs || !atomic_rows_of_part(a, r / kRowParts, r % kRowParts, &r0, &r1)) return;
+    const uint32_t row4 = (uint32_t)(a.nh * a.hd) / 4;
+    typedef T t4 __attribute__((ext_vector_type(4)));
+    const f32x4* src = reinterpret_cast<const f32x4*>(a.grad_value) + ((size_t)b * a.nk + r0) * row4;
+    t4* dst = reinterpret_cast<t4*>(a.grad_value_t) + ((size_t)b * a.nk + r0) * row4;
+    const uint32_t n4 = (uint32_t)(r1 - r0) * row4;
+    for (uint32_t i = threadIdx.x; i < n4; i += blockDim.x) {
+        const f32x4 v = src[i];
+        dst[i] = t4{from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])};
+    }
+}
+
+hipError_t launch_round_rows(int dtype, const KArgs& a, hipStream_t stream)
+{
+    const int64_t grid = (int64_t)a.bs * (a.tbl_stride - 1) * kRowParts;
+    if (grid <= 0 || grid >= (int64_t(1) << 31)) return hipErrorInvalidConfiguration;
+    if (dtype == MXD_DTYPE_F16)
+        hipLaunchKernelGGL(msda_round_rows_kernel<f16_t>, dim3((unsigned)grid), dim3(256), 0, stream, a);
+    else if (dtype == MXD_DTYPE_BF16)
+        hipLaunchKernelGGL(msda_round_rows_kernel<bf16_t>, dim3((unsigned)grid), dim3(256), 0, stream, a);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
 }
 
 // deformable aggregation: grad_location[i] = sum over heads of the per-head partial images

@@ -39,7 +39,6 @@
 
 namespace mxd {
 
-constexpr int kLpp = 8;  // lanes per pixel row = pixels per lane group
 constexpr int kWalk = 2; // lists a lane group walks together, one entry of each per trip
 
 // Work item table, evaluated identically by every workgroup.
@@ -78,17 +77,11 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
         const int32_t H = L.x, W = L.y, base = L.z;
         int32_t P;
         level_tile_count(H, W, base, a.nk, &P);
-        // two pair records per sample, spread evenly over the tiles of the level
-        const int64_t expect = (2 * (int64_t)a.nq * a.np) / nt;
-        int64_t chunks = (expect + t.target - 1) / t.target;
-        if (chunks < 1) chunks = 1;
-        if (chunks > t.max_chunks) chunks = t.max_chunks;
-        if (chunks > a.nwg) chunks = a.nwg;
-        const int32_t wpc = (int32_t)((a.nwg + chunks - 1) / chunks);  // first-kernel workgroups per chunk
-        chunks = (a.nwg + wpc - 1) / wpc;
-        const int32_t n = nt * (int32_t)chunks;
+        int32_t wpc;  // first-kernel workgroups per chunk
+        const int32_t chunks = level_tile_chunks(a, nt, &wpc);
+        const int32_t n = nt * chunks;
         if (item < first + n) {
-            const int32_t ti = (item - first) / (int32_t)chunks, ci = (item - first) % (int32_t)chunks;
+            const int32_t ti = (item - first) / chunks, ci = (item - first) % chunks;
             out->level = l;
             out->H = H;
             out->W = W;
@@ -172,6 +165,8 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     const int nused = copies * npx_pad;              // slots that stand for a pixel of the tile
     const int nspare = kTilePx - nused;              // slots free for extra lists
     const bool can_split = nspare >= kLpp;
+    // (owned && !can_split is what tile_stored_directly() says of this tile)
+    const bool direct_t = a.sparse != 0 && a.grad_value_t != nullptr && owned && !can_split;
     typedef uint16_t __attribute__((may_alias)) u16_alias;  // halves of LDS words that are also accessed whole
     u16_alias* slot_info16 = reinterpret_cast<u16_alias*>(slot_info);
     bool first_round = true;                         // (of the first channel pass)
@@ -484,6 +479,13 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                             float* d1 = reinterpret_cast<float*>(dst);
 #pragma unroll
                             for (int c = 0; c < 4; ++c) unsafeAtomicAdd(d1 + c, v[c]);
+                        } else if (sizeof(T) == 2 && direct_t) {
+                            // 16-bit dtypes: nobody else adds to this row, so it goes to the caller's tensor at once
+                            // (the fp32 image keeps only the rows that receive atomic additions)
+                            typedef T t4 __attribute__((ext_vector_type(4)));
+                            const t4 r = {from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])};
+                            *reinterpret_cast<t4*>(static_cast<T*>(a.grad_value_t) + (size_t)wk.b * (a.gbatch_bytes / 4) +
+                                                   (int64_t)(it.p0 + px) * row_pitch + (int64_t)wk.h * hd + my_ch) = r;
                         } else {
                             if (t.accumulate) v += *dst;
                             *dst = v;

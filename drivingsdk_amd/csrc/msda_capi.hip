@@ -23,6 +23,7 @@ hipError_t launch_backward(int dtype, const KArgs& a, bool scatter, hipStream_t 
 hipError_t launch_gradv_tiles(int dtype, const KArgs& a, const TileArgs& t, hipStream_t stream);
 hipError_t launch_fill_zero(float* p, size_t n, hipStream_t stream);
 hipError_t launch_round(int dtype, const float* src, void* dst, size_t n, hipStream_t stream);
+hipError_t launch_round_rows(int dtype, const KArgs& a, hipStream_t stream);
 hipError_t launch_sum_heads(int dtype, const float* part, void* dst, size_t n, int nh, hipStream_t stream);
 }  // namespace mxd
 
@@ -79,6 +80,10 @@ struct Tuning {
     int fwd_cu_wgs;      // MXD_MSDA_FWD_CU_WGS: its workgroups per (batch, head), 0 = chosen here
     int bwd_fill_kernel; // MXD_MSDA_BWD_FILL_KERNEL: 1 = zero-fill by a kernel of its own
     int tile_order;      // MXD_MSDA_TILE_ORDER: 1 = work items of the tile pass batch-major, 0 = item-major, -1 = chosen here
+    int bwd_sparse;      // MXD_MSDA_BWD_SPARSE: 0 = zero-fill (and, for 16-bit dtypes, round) the whole fp32 image of
+                         // grad_value, 1 = only the rows that receive atomic additions
+    int bwd_lane_bytes;  // MXD_MSDA_BWD_LANE_BYTES: most bytes of a row one lane of the first backward kernel loads
+                         // (16, 8, 4), 0 = chosen here
 };
 Tuning g_tuning;
 std::once_flag g_tuning_once;
@@ -98,6 +103,8 @@ void read_tuning()
     t.fwd_cu_wgs = env_int("MXD_MSDA_FWD_CU_WGS", 0);
     t.bwd_fill_kernel = env_int("MXD_MSDA_BWD_FILL_KERNEL", 0);
     t.tile_order = env_int("MXD_MSDA_TILE_ORDER", -1);
+    t.bwd_lane_bytes = env_int("MXD_MSDA_BWD_LANE_BYTES", 0);
+    t.bwd_sparse = env_int("MXD_MSDA_BWD_SPARSE", 1);
     g_tuning = t;
 }
 
@@ -228,6 +235,19 @@ void row_geometry(int es, int64_t hd, int align_bytes, int* vec_out, int* lpr_ou
     *npass_out = npass;
 }
 
+// Most bytes of a row that one lane of the first backward kernel loads.
+int backward_lane_bytes(int dtype, const Dims& d)
+{
+    const int v = tuning().bwd_lane_bytes;
+    if (v == 4 || v == 8 || v == 16) return v;
+    // Rows of 33 to 64 bytes: 8 lanes of 8 bytes per row rather than 4 lanes of 16.  With 16 units per wavefront the
+    // staging strips of a workgroup take 51 KiB of LDS, which leaves 3 wavefronts per SIMD, and a lane stages four
+    // samples of which it keeps two in registers (measured, encoder shape in float16 / bfloat16: backward 322 -> 300 us;
+    // BEVFormer shape in float16 1114 -> 1075 us; with rows of 256 bytes halving the lane width costs 10 %).
+    const int64_t row = d.hd * elem_size(dtype);
+    return (row > 32 && row <= 64) ? 8 : 16;
+}
+
 // How the backward pass is laid out for a problem size: whether grad_value goes through the
 // tile-ownership pass (and then the hand-over buffers between its two kernels) or through
 // global atomics, and where things live in the caller's workspace.
@@ -239,7 +259,9 @@ void row_geometry(int es, int64_t hd, int align_bytes, int* vec_out, int* lpr_ou
 static int64_t bwd_tile_q(int dtype, const Dims& d)
 {
     // (units with very many samples -- deformable aggregation's 312 -- measured 1 to 2 % better with 64)
-    const int64_t least = (d.hd * elem_size(dtype) <= 64 || d.nl * d.np >= 256) ? 64 : 32;
+    int vec, lpr, npass;
+    row_geometry(elem_size(dtype), d.hd, backward_lane_bytes(dtype, d), &vec, &lpr, &npass);
+    const int64_t least = (mxd::kWave / lpr > 8 || d.nl * d.np >= 256) ? 64 : 32;
     const int v = tuning().bwd_tile_q;
     if (v == 32 || v == 64 || v == 128 || v == 256) return v < least ? least : v;
     // about 512 samples per workgroup for rows of up to 128 bytes, 1024 for longer ones (measured: 32 queries of 16
@@ -275,7 +297,7 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
     const int64_t tbl = d.bs * d.nh * L.nwg * L.tbl_stride * 4;
     // dynamic LDS of the first kernel with the most units per wavefront the row can have (16-byte aligned pointers)
     int vec, lpr, npass;
-    row_geometry(elem_size(dtype), d.hd, 16, &vec, &lpr, &npass);
+    row_geometry(elem_size(dtype), d.hd, backward_lane_bytes(dtype, d), &vec, &lpr, &npass);
     const size_t lds = backward_lds_bytes(mxd::kWave / lpr, 4, true, L.tbl_stride);
     L.tiles = tuning().bwd_atomic == 0 &&
               L.tbl_stride <= 4096 &&                      // counters of the first kernel live in LDS ...
@@ -341,6 +363,20 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
     t->grid = (uint32_t)grid;
     t->block = mxd::kTilePx;
     return MXD_OK;
+}
+
+// Tile mode: how the fp32 image of grad_value gets its zeros and how its rows reach the caller's tensor.  Tiles that
+// one workgroup of the tile pass owns store their rows once; when the rows can be written in 16-byte pieces only the
+// other rows (those that receive atomic additions) are zero-filled, and for 16-bit dtypes the owner stores rounded rows
+// straight into the caller's tensor, so that only those other rows go through the fp32 image and the rounding pass.
+void plan_image(mxd::KArgs* a, mxd::TileArgs* t, bool half, bool accumulate, float* image, void* grad_value, int64_t hd)
+{
+    a->tile_target = t->target;
+    a->tile_max_chunks = t->max_chunks;
+    t->store_vec = (hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
+    a->sparse = tuning().bwd_sparse != 0 && tuning().bwd_fill_kernel == 0 && t->store_vec == 4 && !accumulate &&
+                (!half || (reinterpret_cast<uintptr_t>(grad_value) & 7u) == 0);
+    a->grad_value_t = (a->sparse && half) ? grad_value : nullptr;
 }
 
 // Bytes of LDS the plain forward sets aside for the rows of the last levels (0: none).  Needs 16-byte lanes.
@@ -469,6 +505,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     if (rc != MXD_OK) return rc;
     const int es = elem_size(dtype);
     int vec, lpr, npass;
+    if (backward && align_bytes > backward_lane_bytes(dtype, d)) align_bytes = backward_lane_bytes(dtype, d);
     row_geometry(es, d.hd, align_bytes, &vec, &lpr, &npass);
     if (!backward && cu_form && *cu_form && level_cache) {
         if (plan_forward_cu(dtype, d, vec, lpr, npass, p, level_cache)) return MXD_OK;
@@ -836,7 +873,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     if (!atomic_mode) {
         rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
         if (rc != MXD_OK) return rc;
-        t.store_vec = (hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
+        plan_image(&a, &t, half, (flags & MXD_BWD_ACCUMULATE) != 0, image, grad_value, hd);
     }
     hipError_t e = hipSuccess;
     // zero-fill of the image: by the first kernel's workgroups when the tile pass is the first to touch it and it
@@ -856,7 +893,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: tile kernel launch failed: %s", who, hipGetErrorString(e));
     }
     if (half) {
-        e = mxd::launch_round(dtype, image, grad_value, n, stream);
+        e = a.sparse ? mxd::launch_round_rows(dtype, a, stream) : mxd::launch_round(dtype, image, grad_value, n, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: rounding launch failed: %s", who, hipGetErrorString(e));
     }
     if (part) {
@@ -1061,7 +1098,7 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     if (!atomic_mode) {
         rc = make_tile_args(d, L, a.plan.vec, 0, &t);
         if (rc != MXD_OK) return rc;
-        t.store_vec = (d.hd % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0) ? 4 : 1;
+        plan_image(&a, &t, half, false, image, grad_mc_ms_feat, d.hd);
     }
     hipError_t e = hipSuccess;
     if (L.tiles && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 && tuning().bwd_fill_kernel == 0)
@@ -1077,7 +1114,7 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: tile kernel launch failed: %s", hipGetErrorString(e));
     }
     if (half) {
-        e = mxd::launch_round(dtype, image, grad_mc_ms_feat, n, stream);
+        e = a.sparse ? mxd::launch_round_rows(dtype, a, stream) : mxd::launch_round(dtype, image, grad_mc_ms_feat, n, stream);
         if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_dagg_backward: rounding launch failed: %s", hipGetErrorString(e));
     }
     e = mxd::launch_sum_heads(dtype, part, grad_sampling_location, (size_t)bs * num_anchors * num_pts * num_cams * 2,

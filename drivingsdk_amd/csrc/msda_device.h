@@ -66,6 +66,11 @@ struct KArgs {
     int32_t nwg;           // workgroups of the first kernel per (batch, head)
     int32_t rec_cap;       // 2 * tile_q * nl * np
     int32_t tbl_stride;    // upper bound of tiles per (batch, head), plus one
+    int32_t tile_target;   // pair records per work item of the tile pass aimed at when a hot tile is split by query range
+    int32_t tile_max_chunks;  // most query chunks a tile is split into
+    int32_t sparse;        // 1: only the rows of the image that receive atomic additions are zero-filled (and, for 16-bit
+                           // dtypes, rounded afterwards): the other rows are stored once by the tile's owner
+    void* grad_value_t;    // 16-bit dtypes with sparse = 1: the caller's grad_value, which receives those stores
     int32_t bs, nk, nh, hd, nl, np, nq;
     int32_t S;             // nl*np: samples per unit that are evaluated
     int32_t S_full;        // nl_attn*np: samples per unit that are stored
@@ -83,6 +88,64 @@ __device__ inline i32x4 load_level(const KArgs& a, int l)
     // (int64 metadata: the low words of little-endian elements, two int32 apart)
     const int sh = a.meta_i64;
     return i32x4{a.shapes[(2 * l) << sh], a.shapes[(2 * l + 1) << sh], a.lsi[l << sh], 0};
+}
+
+// ---- tiles of the grad_value pass, as every kernel of the backward sees them ---------------------------------------
+constexpr int kLpp = 8;        // lanes per pixel row = pixels per lane group of the tile pass
+constexpr int kRowParts = 16;  // pieces a tile's rows are cut into for the zero-fill and the rounding
+
+// Query chunks the tiles of a level with `nt` tiles are split into by the tile pass; *wpc: workgroups of the first
+// kernel per chunk.
+__device__ inline int32_t level_tile_chunks(const KArgs& a, int32_t nt, int32_t* wpc)
+{
+    // two pair records per sample, spread evenly over the tiles of the level
+    const int64_t expect = (2 * (int64_t)a.nq * a.np) / nt;
+    int64_t chunks = (expect + a.tile_target - 1) / a.tile_target;
+    if (chunks < 1) chunks = 1;
+    if (chunks > a.tile_max_chunks) chunks = a.tile_max_chunks;
+    if (chunks > a.nwg) chunks = a.nwg;
+    *wpc = (int32_t)((a.nwg + chunks - 1) / chunks);
+    return (int32_t)((a.nwg + *wpc - 1) / *wpc);
+}
+
+// A tile of `npx` pixels whose rows its one workgroup of the tile pass stores directly: no other workgroup adds to
+// them (the tile is not split by query range and is too full to be held in copies or to have slots left for extra
+// lists), except to the tile's first pixel, which also receives the right halves of pairs that start on the last
+// pixel of the tile before it.
+__device__ inline bool tile_stored_directly(int32_t chunks, int32_t npx)
+{
+    return chunks == 1 && kTilePx - ((npx + kLpp - 1) / kLpp * kLpp) < kLpp;
+}
+
+// Rows (pixels of a batch element) [*r0, *r1) of piece `part` (< kRowParts) of tile `tile` of a batch element that
+// receive atomic additions in the tile pass; false when there is no such tile.  Tiles are numbered level by level as
+// in the first kernel and the tile pass.
+__device__ inline bool atomic_rows_of_part(const KArgs& a, int32_t tile, int32_t part, int32_t* r0, int32_t* r1)
+{
+    int32_t first = 0;
+    for (int l = 0; l < a.nl; ++l) {
+        const i32x4 L = load_level(a, l);
+        int32_t P;
+        const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, &P);
+        if (first + nt > a.tbl_stride - 1) continue;  // (a level that does not fit the run table has no tiles)
+        if (tile < first + nt) {
+            const int32_t ti = tile - first;
+            const int32_t p0 = L.z + ti * kTilePx;
+            const int32_t npx = (P - ti * kTilePx) < kTilePx ? (P - ti * kTilePx) : kTilePx;
+            int32_t wpc;
+            if (tile_stored_directly(level_tile_chunks(a, nt, &wpc), npx)) {
+                *r0 = p0;
+                *r1 = part == 0 ? p0 + 1 : p0;
+            } else {
+                constexpr int per = kTilePx / kRowParts;
+                *r0 = p0 + (part * per < npx ? part * per : npx);
+                *r1 = p0 + ((part + 1) * per < npx ? (part + 1) * per : npx);
+            }
+            return true;
+        }
+        first += nt;
+    }
+    return false;
 }
 
 // Where a kernel takes the location and the weight of sample s of unit (b, q, h) from.

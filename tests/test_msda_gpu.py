@@ -755,15 +755,16 @@ def test_random_small_problems_cu_form(gpu_device, monkeypatch, seed):
 
 
 def test_backward_with_more_tiles_than_the_lds_bookkeeping_holds(gpu_device):
-    """One level of 2.09 M pixels and 64-byte rows (a 1080x1920 grid-sampler-like input): the per-tile counters of the
+    """One level of 2.09 M pixels and 32-byte rows (a 1080x1920 grid-sampler-like input): the per-tile counters of the
     first backward kernel would not fit the LDS next to 16 units' staging strips, so the launcher takes the
     one-kernel form with global atomics.  Gradients against the oracle."""
     g = torch.Generator().manual_seed(2090)
     levels = ((1100, 1900),)
     shapes, lsi = workloads.level_tensors(levels)
     nk = 1100 * 1900
-    bs, nq, nh, hd, npts = 1, 2000, 1, 16, 4
+    bs, nq, nh, hd, npts = 1, 2000, 1, 8, 4
     plan = _lib.make_plan(1, 0, bs, nk, nh, hd, 1, 1, nq, npts)
+    assert plan.units_per_wave == 16
     assert plan.lds_bytes <= 64 * 1024 and plan.iters == 1      # (the atomic form: one iteration per wavefront)
     assert _lib.load().mxd_msda_backward_workspace_bytes(0, bs, nk, nh, hd, 1, 1, nq, npts) == 0
     inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g), shapes, lsi,
