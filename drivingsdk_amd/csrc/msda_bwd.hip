@@ -119,10 +119,15 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         smem + kMaxLevels * sizeof(i32x4) +
         (size_t)a.plan.waves_per_block * a.plan.units_per_wave * (kChunkStride * sizeof(Entry) + kChunk * sizeof(f32x4)));
     int32_t* cursor = tile_first + kMaxLevels;  // [tbl_stride] counts, then next free position per tile
-    u32x4* slab = nullptr;
+    uint32_t* slab = nullptr;
     const int entries = U * kChunk;
     // ---- per unit: the grad_out row in the value-load layout and, for the fused form, the softmax terms ----
     float gv[NPASS][VEC];
+    // 16-bit rows: the same row as packed pairs, for dot products that multiply two pairs of 16-bit elements exactly
+    // and add them to a float32 sum in one instruction (v_dot2c_f32_f16 / v_dot2c_f32_bf16)
+    constexpr bool kDot2 = sizeof(T) == 2 && VEC % 2 == 0;
+    constexpr int kPairs = kDot2 ? VEC / 2 : 1;
+    uint32_t gpk[NPASS][kPairs];
     auto unit_prologue = [&](int q0) {
         // grad_out row of this lane's unit in the value-load layout (for the dots)
         const int qg = q0 + g;
@@ -136,6 +141,12 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             } else {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) gv[p][e] = 0.0f;
+            }
+            if constexpr (kDot2) {
+                typedef T t2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+                for (int e = 0; e < kPairs; ++e)
+                    gpk[p][e] = __builtin_bit_cast(uint32_t, t2{from_f32<T>(gv[p][2 * e]), from_f32<T>(gv[p][2 * e + 1])});
             }
         }
 
@@ -276,7 +287,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     };
     if constexpr (!SCATTER) {
         const int64_t wg_row = ((int64_t)wk.b * a.nh + wk.h) * a.nwg + wk.q_begin / a.plan.tile_q;
-        slab = a.rec + wg_row * a.rec_cap;
+        slab = a.rec + wg_row * a.rec_cap * kRecDwords;
         if (threadIdx.x == 0) {
             // the run table has room for tbl_stride - 1 tiles, which is every tile when the levels do not
             // overlap; a level that does not fit (malformed shapes) is left out of grad_value: -1
@@ -380,9 +391,16 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                                         (size_t)(unit & (U - 1)) * (kChunkStride * sizeof(Entry))) +
                (pos & 31);
     };
+    // (records take a 16-byte slot in LDS and 12 bytes in the slab)
+    typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+    const __amdgpu_buffer_rsrc_t sres = make_rsrc(slab, SCATTER ? 0u : (uint32_t)a.rec_cap * (kRecDwords * 4u));
+    auto store_record = [&](int pos, const u32x4 rec) {
+        // (non-temporal: the records are read by the next kernel and should not push value rows out of L2)
+        __builtin_amdgcn_raw_buffer_store_b96(u32x3{rec.x, rec.y, rec.z}, sres, (uint32_t)pos * (kRecDwords * 4u), 0, 2);
+    };
     auto copy_records_out = [&]() {
         const int total = cursor[a.tbl_stride - 1];  // (exclusive prefix: the entry after the last tile holds the sum)
-        for (int i = threadIdx.x; i < total; i += blockDim.x) __builtin_nontemporal_store(*rec_lds(i), slab + i);
+        for (int i = threadIdx.x; i < total; i += blockDim.x) store_record(i, *rec_lds(i));
     };
 
     for (int it = 0; it < a.plan.iters; ++it) {
@@ -420,10 +438,17 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         for (int k = 0; k < NC; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
 #pragma unroll
                         for (int k = 0; k < NC; ++k) {
-                            float v[VEC];
-                            RowIO<T, VEC>::unpack(raw[k], v);
+                            if constexpr (kDot2) {
+                                uint32_t words[kPairs];
+                                __builtin_memcpy(words, &raw[k], sizeof(words));
 #pragma unroll
-                            for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
+                                for (int e = 0; e < kPairs; ++e) d[k] = dot2_acc<T>(words[e], gpk[p][e], d[k]);
+                            } else {
+                                float v[VEC];
+                                RowIO<T, VEC>::unpack(raw[k], v);
+#pragma unroll
+                                for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
+                            }
                         }
                     }
                     f32x4 dsum = {0.f, 0.f, 0.f, 0.f};
@@ -625,10 +650,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                         if (rec_keep[r]) {
                             const int32_t pos =
                                 atomicAdd(&cursor[tile_first[rec_l] + ((rec_key[r] - lvl[rec_l].z) >> kTilePxLog2)], 1);
-                            const u32x4 rec = {(uint32_t)rec_key[r], (uint32_t)q, __builtin_bit_cast(uint32_t, rec_wa[r]),
-                                               __builtin_bit_cast(uint32_t, rec_wb[r])};
+                            const uint32_t in_tile = (uint32_t)(rec_key[r] - lvl[rec_l].z) & (uint32_t)(kTilePx - 1);
+                            const u32x4 rec = {in_tile | ((uint32_t)(q - wk.q_begin) << kTilePxLog2),
+                                               __builtin_bit_cast(uint32_t, rec_wa[r]), __builtin_bit_cast(uint32_t, rec_wb[r]), 0u};
                             if (rec_in_lds) *rec_lds(pos) = rec;
-                            else __builtin_nontemporal_store(rec, slab + pos);
+                            else store_record(pos, rec);
                         }
                     }
                 }

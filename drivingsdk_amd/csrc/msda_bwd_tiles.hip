@@ -177,7 +177,10 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     const T* gout = static_cast<const T*>(a.grad_out);
     const int64_t bh = (int64_t)wk.b * a.nh + wk.h;
     const uint32_t* tbl = a.tbl + bh * a.nwg * a.tbl_stride + it.tile;
-    const u32x4* rec = a.rec + bh * a.nwg * a.rec_cap;
+    // the records of this (batch, head) as a bound buffer (the layout keeps them below 4 GiB)
+    typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+    const __amdgpu_buffer_rsrc_t rres = make_rsrc(a.rec + bh * a.nwg * a.rec_cap * kRecDwords,
+                                                  (uint32_t)a.nwg * (uint32_t)a.rec_cap * (kRecDwords * 4u));
     // runs of this wavefront: workgroups it.w0 + wave, + NW, + 2 NW, ... of the first kernel
     const int nruns = (it.w1 - it.w0 - wave + NW - 1) / NW;  // <= 0: none
 
@@ -219,7 +222,12 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
 #pragma unroll
                 for (int step = kWave / 2; step > 0; step >>= 1)
                     if (run_pre[r + step] <= (uint32_t)i) r += step;
-                ahead = __builtin_nontemporal_load(rec + (run_src[r] + ((uint32_t)i - run_pre[r])));
+                // (one 12-byte load, non-temporal: the records are read once)
+                const u32x3 v = __builtin_bit_cast(
+                    u32x3, __builtin_amdgcn_raw_buffer_load_b96(rres, (run_src[r] + ((uint32_t)i - run_pre[r])) * (kRecDwords * 4u), 0, 2));
+                // (run r of the current group comes from workgroup it.w0 + wave + NW * (rg - 64 + r) of the first kernel;
+                //  its records name queries relative to that workgroup's first one)
+                ahead = u32x4{v.x, v.y, v.z, (uint32_t)(it.w0 + wave + NW * (rg - kWave + r)) * (uint32_t)a.plan.tile_q};
             }
         };
         bool counted = false;    // this wavefront has reported the end of its work
@@ -272,10 +280,11 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 float wb = 0.f;
                 // (a record that does not belong to this tile or names no query of the batch element is dropped:
                 // the run table and the records are only as good as the workspace the caller hands over)
-                if (have && (uint32_t)((int)rc.x - it.p0) < (uint32_t)npx && rc.y < (uint32_t)a.nq) {
-                    const uint32_t kx = rc.x, qx = rc.y, ya = rc.z, za = rc.w;
-                    q = qx;
-                    const int pl = (int)kx - it.p0;
+                const uint32_t rkey = rc.x, rq0 = rc.w;
+                if (have && (rkey & (uint32_t)(kTilePx - 1)) < (uint32_t)npx && rq0 + (rkey >> kTilePxLog2) < (uint32_t)a.nq) {
+                    const uint32_t ya = rc.y, za = rc.z;
+                    q = rq0 + (rkey >> kTilePxLog2);
+                    const int pl = (int)(rkey & (uint32_t)(kTilePx - 1));
                     const float wa = __builtin_bit_cast(float, ya);
                     wb = __builtin_bit_cast(float, za);
                     const int copy_off = (int)(q & (uint32_t)(copies - 1)) * npx_pad;

@@ -303,11 +303,11 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
               L.tbl_stride <= 4096 &&                      // counters of the first kernel live in LDS ...
               lds <= 64 * 1024 &&                          // ... and its strips and counters fit the default limit
               tbl <= (int64_t(1) << 28) &&                 // run table of at most 256 MiB
-              L.nwg * L.rec_cap < (int64_t(1) << 31) &&    // 32-bit record indices within a (batch, head)
+              L.nwg * L.rec_cap * (mxd::kRecDwords * 4) < (int64_t(1) << 32) &&  // 32-bit byte offsets of the records of a (batch, head)
               d.nq * d.nh * d.hd * 4 < (int64_t(1) << 31); // grad_output rows addressed with 32-bit byte offsets
     if (L.tiles) {
         L.tbl_bytes = ((size_t)tbl + 255) & ~(size_t)255;
-        L.rec_bytes = (size_t)d.bs * d.nh * L.nwg * L.rec_cap * 16;
+        L.rec_bytes = ((size_t)d.bs * d.nh * L.nwg * L.rec_cap * (mxd::kRecDwords * 4) + 255) & ~(size_t)255;
     }
     if (elem_size(dtype) == 2) L.image_bytes = (size_t)d.bs * d.nk * d.nh * d.hd * 4;
     L.total = L.tbl_bytes + L.rec_bytes + L.image_bytes;
@@ -846,7 +846,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     a.grad_out = grad_output;
     a.grad_value = image;
     a.tbl = reinterpret_cast<uint32_t*>(ws);
-    a.rec = reinterpret_cast<mxd::u32x4*>(ws + L.tbl_bytes);
+    a.rec = reinterpret_cast<uint32_t*>(ws + L.tbl_bytes);
     a.nwg = (int32_t)L.nwg;
     a.rec_cap = (int32_t)L.rec_cap;
     a.tbl_stride = (int32_t)L.tbl_stride;
@@ -1084,7 +1084,7 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     a.grad_out = grad_output;
     a.grad_value = image;
     a.tbl = reinterpret_cast<uint32_t*>(ws);
-    a.rec = reinterpret_cast<mxd::u32x4*>(ws + L.tbl_bytes);
+    a.rec = reinterpret_cast<uint32_t*>(ws + L.tbl_bytes);
     a.nwg = (int32_t)L.nwg;
     a.rec_cap = (int32_t)L.rec_cap;
     a.tbl_stride = (int32_t)L.tbl_stride;

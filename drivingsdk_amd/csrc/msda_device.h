@@ -60,8 +60,9 @@ struct KArgs {
     // first kernel (tile_q queries of one (batch, head)) owns a slab of rec_cap pair records,
     // which it fills sorted by tile; row [w] of the table holds the start of every tile's run
     // inside slab w (tbl_stride entries, the last used one being the total).
-    // record = {pixel index, query, weight of that pixel, weight of the pixel to its right}
-    u32x4* rec;            // [bs*nh][nwg][rec_cap]
+    // record (12 bytes) = {pixel within its tile | query within the workgroup << kTilePxLog2, weight of that pixel,
+    //                      weight of the pixel to its right}
+    uint32_t* rec;         // [bs*nh][nwg][rec_cap] records of kRecDwords dwords
     uint32_t* tbl;         // [bs*nh][nwg][tbl_stride]
     int32_t nwg;           // workgroups of the first kernel per (batch, head)
     int32_t rec_cap;       // 2 * tile_q * nl * np
@@ -91,6 +92,7 @@ __device__ inline i32x4 load_level(const KArgs& a, int l)
 }
 
 // ---- tiles of the grad_value pass, as every kernel of the backward sees them ---------------------------------------
+constexpr int kRecDwords = 3;  // dwords of a pair record
 constexpr int kLpp = 8;        // lanes per pixel row = pixels per lane group of the tile pass
 constexpr int kRowParts = 16;  // pieces a tile's rows are cut into for the zero-fill and the rounding
 
@@ -225,6 +227,18 @@ template <typename T>
 __device__ inline T from_f32(float v)
 {
     return (T)v;
+}
+
+// acc + a.lo * b.lo + a.hi * b.hi for two packed pairs of 16-bit elements, the products and the sum in float32.
+template <typename T>
+__device__ inline float dot2_acc(uint32_t a, uint32_t b, float acc)
+{
+    static_assert(sizeof(T) == 2, "packed pairs of 16-bit elements");
+    typedef T t2 __attribute__((ext_vector_type(2)));
+    if constexpr (std::is_same<T, f16_t>::value)
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(t2, a), __builtin_bit_cast(t2, b), acc, false);
+    else
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(t2, a), __builtin_bit_cast(t2, b), acc, false);
 }
 
 // One coordinate of a sampling location.  Geometric kernel attention carries pixel indices: they are float32 whatever

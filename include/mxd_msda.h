@@ -168,7 +168,7 @@ int mxd_msda_fused_backward(const void* value, const int32_t* spatial_shapes, co
 
 /* Bytes of scratch mxd_msda_backward needs (0 if the sizes are invalid, and for float32 sizes
  * that take the one-kernel path with global atomics).  It holds the hand-over between the two
- * backward kernels -- a table of run starts and two 16-byte records per sample, written
+ * backward kernels -- a table of run starts and two 12-byte records per sample, written
  * sorted by tile by the first kernel and streamed by the second -- and, for fp16/bf16, an
  * fp32 image of grad_value (bs*nk*nh*hd*4) that the sums are formed in before one rounding
  * pass (the reference keeps the same fp32 buffer, MultiScaleDeformableAttn.cpp:93,103-113;

@@ -113,12 +113,13 @@ def test_workspace_size():
     lib = _lib.load()
     # bs 2, nk 100, nh 8, hd 32, nl 4, nq 50, np 3.  The first backward kernel runs 32-query workgroups for rows
     # of more than 32 bytes (eight units per wavefront: two workgroups per (batch, head) here) and 64-query ones
-    # for shorter rows (sixteen units: one); a workgroup's slab holds two pair records (16 B) per sample; the run
+    # for shorter rows (sixteen units: one); a workgroup's slab holds two pair records (12 B) per sample (the
+    # record area is padded to 256 bytes); the run
     # table has one column per possible tile (nk // 512 + nl) plus one per workgroup, padded to 256 bytes
     def expect(tile_q):
         nwg = -(-50 // tile_q)
         table = -(-(2 * 8 * nwg * (100 // 512 + 4 + 1) * 4) // 256) * 256
-        return table + 2 * 8 * nwg * (2 * tile_q * 4 * 3) * 16
+        return table + -(-(2 * 8 * nwg * (2 * tile_q * 4 * 3) * 12) // 256) * 256
     image = 2 * 100 * 8 * 32 * 4
     assert lib.mxd_msda_backward_workspace_bytes(0, 2, 100, 8, 32, 4, 4, 50, 3) == expect(32)
     assert lib.mxd_msda_backward_workspace_bytes(1, 2, 100, 8, 32, 4, 4, 50, 3) == expect(32) + image
