@@ -240,9 +240,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 en.off[k] = sm.cvalid[k] ? (uint32_t)sm.pix[k] * a.pitch_bytes : kInvalidCorner;
-                en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
+                if constexpr (SCATTER) en.w[k] = sm.valid ? sm.w[k] * aw : 0.0f;
             }
-            stage[u * kChunkStride + sl] = en;
+            // (the weights are read by the scatter of the one-kernel form only)
+            if constexpr (SCATTER) stage[u * kChunkStride + sl] = en;
+            else *reinterpret_cast<u32x4*>(stage[u * kChunkStride + sl].off) = u32x4{en.off[0], en.off[1], en.off[2], en.off[3]};
             if (ks < kKeep) {
                 keep_lw[ks % kKeepRegs] = sm.lw;
                 keep_lh[ks % kKeepRegs] = sm.lh;
