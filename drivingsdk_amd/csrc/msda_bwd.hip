@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     if constexpr (!SCATTER) {
         // this workgroup's share of the zero-fill of the image (every workgroup of the launch takes one, also those
         // without work): the stores ride along with this kernel instead of taking a launch of their own
-        if (a.fill_n4 != 0 && a.sparse != 0) {
+        if (a.fill_n4 != 0 && a.sparse != 0 && levels_tile_the_keys(a)) {
             // only the rows that receive atomic additions in the tile pass (tiles split by query range, small tiles,
             // and the first pixel of every other tile); a row of the image is nh*hd floats, a multiple of 16 bytes here
             const int32_t tiles = a.tbl_stride - 1;  // (bound: pieces of tiles that do not exist are skipped)
@@ -713,11 +713,23 @@ template <typename T>
 __global__ __launch_bounds__(256) void msda_round_rows_kernel(const KArgs a)
 {
     const int32_t tiles = a.tbl_stride - 1;
+    const uint32_t row4 = (uint32_t)(a.nh * a.hd) / 4;
+    typedef T t4 __attribute__((ext_vector_type(4)));
+    if (!levels_tile_the_keys(a)) {
+        // every row went through the fp32 image: the workgroups round it between them
+        const uint64_t n4 = (uint64_t)a.bs * a.nk * row4, per = (n4 + gridDim.x - 1) / gridDim.x;
+        const uint64_t lo = (uint64_t)blockIdx.x * per, hi = lo + per < n4 ? lo + per : n4;
+        const f32x4* src = reinterpret_cast<const f32x4*>(a.grad_value);
+        t4* dst = reinterpret_cast<t4*>(a.grad_value_t);
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+            const f32x4 v = src[i];
+            dst[i] = t4{from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])};
+        }
+        return;
+    }
     const int32_t b = (int32_t)(blockIdx.x / (uint32_t)(tiles * kRowParts)), r = (int32_t)(blockIdx.x % (uint32_t)(tiles * kRowParts));
     int32_t r0, r1;
     if (b >= a.bs || !atomic_rows_of_part(a, r / kRowParts, r % kRowParts, &r0, &r1)) return;
-    const uint32_t row4 = (uint32_t)(a.nh * a.hd) / 4;
-    typedef T t4 __attribute__((ext_vector_type(4)));
     const f32x4* src = reinterpret_cast<const f32x4*>(a.grad_value) + ((size_t)b * a.nk + r0) * row4;
     t4* dst = reinterpret_cast<t4*>(a.grad_value_t) + ((size_t)b * a.nk + r0) * row4;
     const uint32_t n4 = (uint32_t)(r1 - r0) * row4;

@@ -47,7 +47,8 @@ struct TileItem {
     int32_t p0, p1;              // pixel range of the tile, relative to the batch element
     int32_t w0, w1;              // range of workgroups of the first kernel whose records are taken
     int32_t tile;                // index of the tile within the (batch, head): column of the run table
-    int32_t exclusive;           // 1: no other workgroup touches this tile
+    int32_t exclusive;           // 1: no other workgroup touches this tile (the item is not split by query range and the
+                                 // levels tile the keys, so that no tile of another level holds the same rows)
 };
 
 // lv_first / lv_nt: scratch of kMaxLevels entries each (first tile and tile count per level).
@@ -66,6 +67,7 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
         lv_nt[l] = fits ? nt : 0;
         if (fits) total += nt;
     }
+    const bool canonical = levels_tile_the_keys(a);
     // Items are numbered from the last level to the first: the coarse levels, whose tiles are
     // split into many long-running items, start first and the short items of the fine levels
     // fill the end of the launch.
@@ -91,7 +93,7 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
             out->w0 = ci * wpc;
             out->w1 = (out->w0 + wpc) < a.nwg ? (out->w0 + wpc) : a.nwg;
             out->tile = lv_first[l] + ti;
-            out->exclusive = chunks == 1;
+            out->exclusive = chunks == 1 && canonical;
             return true;
         }
         first += n;

@@ -119,6 +119,27 @@ __device__ inline bool tile_stored_directly(int32_t chunks, int32_t npx)
     return chunks == 1 && kTilePx - ((npx + kLpp - 1) / kLpp * kLpp) < kLpp;
 }
 
+// Whether the levels tile the keys exactly and in order -- the first level starts at key 0, every other one where the
+// one before it ends, the last one ends at key nk -- and all their tiles fit the run table.  Only then is every row of
+// grad_value covered by exactly one tile, which is what lets the owner of a tile store its rows (instead of adding to
+// them) and lets the rows that nobody adds to go without zeros.  level_start_index is the caller's: for any other
+// layout (keys that no level covers, levels out of order or overlapping) every row is zero-filled and every tile adds
+// its sums with atomics.
+__device__ inline bool levels_tile_the_keys(const KArgs& a)
+{
+    int64_t next = 0;
+    int32_t tiles = 0;
+    for (int l = 0; l < a.nl; ++l) {
+        const i32x4 L = load_level(a, l);
+        if (L.x <= 0 || L.y <= 0 || (int64_t)L.z != next) return false;
+        const int64_t px = (int64_t)L.x * L.y;
+        next += px;
+        if (next > a.nk) return false;
+        tiles += (int32_t)((px + kTilePx - 1) >> kTilePxLog2);
+    }
+    return next == a.nk && tiles <= a.tbl_stride - 1;
+}
+
 // Rows (pixels of a batch element) [*r0, *r1) of piece `part` (< kRowParts) of tile `tile` of a batch element that
 // receive atomic additions in the tile pass; false when there is no such tile.  Tiles are numbered level by level as
 // in the first kernel and the tile pass.

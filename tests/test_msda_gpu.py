@@ -771,3 +771,46 @@ def test_backward_with_more_tiles_than_the_lds_bookkeeping_holds(gpu_device):
                                torch.rand(bs, nq, nh, 1, npts, 2, generator=g) * 1.02 - 0.01,
                                torch.rand(bs, nq, nh, 1, npts, generator=g), torch.randn(bs, nq, nh * hd, generator=g))
     print(_check_all(inp, gpu_device, FWD_FP32, BWD_FP32))
+
+
+_LAYOUTS = {
+    # name: (level shapes, level_start_index, num_keys)
+    "keys_behind_the_last_level": (((40, 30), (20, 15)), (0, 1200), 1200 + 300 + 777),
+    "gap_between_levels": (((40, 30), (20, 15)), (0, 1500), 1800 + 50),
+    "descending_starts": (((40, 30), (20, 15)), (300, 0), 1500),
+    "overlapping_levels": (((40, 30), (20, 15)), (0, 1000), 1300),
+    "first_level_does_not_start_at_zero": (((40, 30), (20, 15)), (600, 1800), 2100),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("layout", sorted(_LAYOUTS))
+@pytest.mark.parametrize("cu", ["0", "1"])
+def test_level_start_indices_that_do_not_tile_the_keys(gpu_device, monkeypatch, layout, dtype, cu):
+    """level_start_index is the caller's: the reference's kernels index value with it as given and add gradients with
+    atomics, so levels may leave keys uncovered, come in any order or overlap (kernels/multi_scale_deformable_attn/
+    op_kernel/multi_scale_deformable_attn_grad.cpp:181-186).  Rows of grad_value that no level covers are exactly zero."""
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=cu)
+    levels, starts, nk = _LAYOUTS[layout]
+    shapes = torch.tensor(levels, dtype=torch.int64)
+    lsi = torch.tensor(starts, dtype=torch.int64)
+    bs, nq, nh, hd, npts = 2, 3100, 3, 32, 4
+    g = torch.Generator().manual_seed(len(layout))
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g).to(dtype), shapes, lsi,
+                               (torch.rand(bs, nq, nh, 2, npts, 2, generator=g) * 1.1 - 0.05).to(dtype),
+                               torch.rand(bs, nq, nh, 2, npts, generator=g).to(dtype),
+                               torch.randn(bs, nq, nh * hd, generator=g).to(dtype))
+    ref = oracle_all(inp)
+    got = run_gpu(inp, gpu_device)
+    tol_f, tol_b = (FWD_FP32, BWD_FP32) if dtype == torch.float32 else (HALF, HALF)
+    for name, g_, r_, tol in zip(("output", "grad_value", "grad_sampling_locations", "grad_attention_weights"), got, ref,
+                                 (tol_f, tol_b, tol_b, tol_b)):
+        if name == "grad_sampling_locations":
+            keep = ~_cell_edge_mask(inp)[..., None]
+            g_, r_ = g_ * keep, np.asarray(r_) * keep
+        assert rel_err(g_, r_) <= tol, (name, rel_err(g_, r_))
+    covered = np.zeros(nk, dtype=bool)
+    for (h, w), s in zip(levels, starts):
+        covered[s:s + h * w] = True
+    assert not np.any(got[1][:, ~covered]), "rows of grad_value outside every level must be exactly zero"

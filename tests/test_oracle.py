@@ -179,6 +179,41 @@ def test_gradients_against_finite_differences():
             np.testing.assert_allclose(grad.reshape(-1)[fi], fd, rtol=2e-5, atol=1e-6, err_msg=name)
 
 
+def test_level_start_index_is_honoured_as_given():
+    """The direct form indexes value with level_start_index as given (the reference: op_kernel/msda.h:428 and the
+    arch35 kernels add the level's start to y*W + x).  Moving the levels around inside value -- other order, a gap, keys
+    that no level covers -- must not change the output, and the gradient of value moves with the levels; uncovered
+    rows get exactly zero.  Pinned against the canonical layout, which the grid_sample formulation pins."""
+    levels = [(7, 5), (4, 6), (3, 3)]
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    g = torch.Generator().manual_seed(31)
+    bs, nq, nh, hd, npts = 2, 9, 2, 3, 4
+    value = torch.randn(bs, nk, nh, hd, generator=g, dtype=torch.float64)
+    loc = torch.rand(bs, nq, nh, 3, npts, 2, generator=g, dtype=torch.float64) * 1.2 - 0.1
+    attn = torch.rand(bs, nq, nh, 3, npts, generator=g, dtype=torch.float64)
+    go = torch.randn(bs, nq, nh * hd, generator=g, dtype=torch.float64)
+    out = orc.direct_forward(value, shapes, lsi, loc, attn)
+    gv, gl, ga = orc.direct_backward(value, shapes, lsi, loc, attn, go)
+    # level 2 first, then five keys nobody uses, level 0, a gap of two, level 1, three keys behind it
+    new_starts = torch.tensor([9 + 5, 9 + 5 + 35 + 2, 0])
+    nk2 = 9 + 5 + 35 + 2 + 24 + 3
+    value2 = torch.full((bs, nk2, nh, hd), 123.0, dtype=torch.float64)
+    for l, (h, w) in enumerate(levels):
+        value2[:, int(new_starts[l]):int(new_starts[l]) + h * w] = value[:, int(lsi[l]):int(lsi[l]) + h * w]
+    out2 = orc.direct_forward(value2, shapes, new_starts, loc, attn)
+    gv2, gl2, ga2 = orc.direct_backward(value2, shapes, new_starts, loc, attn, go)
+    np.testing.assert_allclose(out2, out, rtol=0, atol=1e-13)
+    np.testing.assert_allclose(gl2, gl, rtol=0, atol=1e-13)
+    np.testing.assert_allclose(ga2, ga, rtol=0, atol=1e-13)
+    covered = np.zeros(nk2, dtype=bool)
+    for l, (h, w) in enumerate(levels):
+        a, b = int(new_starts[l]), int(lsi[l])
+        np.testing.assert_allclose(np.asarray(gv2)[:, a:a + h * w], np.asarray(gv)[:, b:b + h * w], rtol=0, atol=1e-13)
+        covered[a:a + h * w] = True
+    assert not np.any(np.asarray(gv2)[:, ~covered])
+
+
 @pytest.mark.parametrize("fill", [float("nan"), float("inf"), float("-inf")])
 def test_nan_inf_known_answer_all_zero(fill):
     """All float inputs NaN or Inf: every output is exactly zero
