@@ -868,7 +868,8 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     const size_t n = (size_t)bs * nk * nh * hd;
     // every step that can fail for the sizes given comes before the first launch
-    const bool atomic_mode = !L.tiles;
+    // (MXD_BWD_ANY_LAYOUT: the one-kernel form with global atomics, which takes level_start_index as it comes)
+    const bool atomic_mode = !L.tiles || (flags & MXD_BWD_ANY_LAYOUT) != 0;
     mxd::TileArgs t;
     if (!atomic_mode) {
         rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
@@ -878,7 +879,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     hipError_t e = hipSuccess;
     // zero-fill of the image: by the first kernel's workgroups when the tile pass is the first to touch it and it
     // can be written in 16-byte pieces, by a kernel of its own otherwise
-    const bool fill_inside = L.tiles && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 &&
+    const bool fill_inside = !atomic_mode && n % 4 == 0 && (reinterpret_cast<uintptr_t>(image) & 15u) == 0 &&
                              tuning().bwd_fill_kernel == 0;
     if (!(flags & MXD_BWD_ACCUMULATE)) {
         if (fill_inside) a.fill_n4 = n / 4;

@@ -17,10 +17,11 @@ pytestmark = pytest.mark.gpu
 
 
 def _cell_edge_mask(inp):
-    """Samples whose pixel coordinate lies within 2^-20 of an integer on either axis.  The
-    location gradient of bilinear interpolation jumps there (it is the slope of the cell the
-    sample falls in), so a float32 and a float64 evaluation may legitimately pick different
-    sides; such samples are left out of the grad_sampling_locations comparison only."""
+    """Samples whose pixel coordinate lies within 2^-20 -- or, where that is more, two float32 units in the last place
+    of the coordinate -- of an integer on either axis.  The location gradient of bilinear interpolation jumps there (it
+    is the slope of the cell the sample falls in; at the border of the image the sample's validity flips), so a
+    float32 and a float64 evaluation may legitimately pick different sides; such samples are left out of the
+    grad_sampling_locations comparison only."""
     loc = inp.sampling_locations.double()
     nl = inp.spatial_shapes.shape[0]
     hw = inp.spatial_shapes.double()
@@ -30,7 +31,11 @@ def _cell_edge_mask(inp):
         h_im = loc[:, :, :, lvl, :, 1] * hw[lvl, 0] - 0.5
         dw, dh = (w_im - w_im.round()).abs(), (h_im - h_im.round()).abs()
         # exactly on an edge is fine: both evaluations are exact there and take the same side
-        near = ((dw > 0) & (dw < 2.0 ** -20)) | ((dh > 0) & (dh < 2.0 ** -20))
+        # (float32 spacing at coordinate c: 2^(floor(log2 |c|) - 23))
+        ulp_w = torch.exp2(torch.floor(torch.log2(w_im.abs().clamp_min(1.0))) - 23.0)
+        ulp_h = torch.exp2(torch.floor(torch.log2(h_im.abs().clamp_min(1.0))) - 23.0)
+        near = ((dw > 0) & (dw < torch.maximum(2.0 * ulp_w, torch.tensor(2.0 ** -20, dtype=torch.float64)))) | \
+               ((dh > 0) & (dh < torch.maximum(2.0 * ulp_h, torch.tensor(2.0 ** -20, dtype=torch.float64))))
         mask[:, :, :, lvl] = near
     return mask.numpy()
 
@@ -52,7 +57,8 @@ def _check_all(inp, device, fwd_tol, bwd_tol, with_grads=True):
         r = np.asarray(r)
         if name == "grad_sampling_locations":
             edge = _cell_edge_mask(inp)
-            assert edge.mean() < 1e-4 or dtype != torch.float32, "too many samples sit on a cell edge for this check to mean anything"
+            # (levels thousands of pixels wide have float32 coordinates spaced 2^-13 apart: up to a thousandth of the samples)
+            assert edge.mean() < 2e-3 or dtype != torch.float32, "too many samples sit on a cell edge for this check to mean anything"
             keep = ~edge[..., None]
             g, r = g * keep, r * keep
             errs["cell_edge_samples"] = int(edge.sum())
@@ -814,3 +820,23 @@ def test_level_start_indices_that_do_not_tile_the_keys(gpu_device, monkeypatch, 
     for (h, w), s in zip(levels, starts):
         covered[s:s + h * w] = True
     assert not np.any(got[1][:, ~covered]), "rows of grad_value outside every level must be exactly zero"
+
+
+def test_any_layout_flag_sums_levels_that_overlap_beyond_the_run_table(gpu_device):
+    """Four levels that overlap so far that they have 17 tiles of 512 pixels between them while value has 3 422 keys
+    (room for 10 in the run table): with MXD_BWD_ANY_LAYOUT the backward takes the form with global atomics, which, like
+    the reference's kernel, takes level_start_index as it comes."""
+    levels, starts, nk = ((56, 48), (10, 20), (58, 55), (58, 18)), (504, 1119, 148, 352), 3422
+    bs, nq, nh, hd, npts = 2, 300, 4, 32, 5
+    g = torch.Generator().manual_seed(77)
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g), torch.tensor(levels), torch.tensor(starts),
+                               torch.rand(bs, nq, nh, 4, npts, 2, generator=g) * 1.2 - 0.1,
+                               torch.rand(bs, nq, nh, 4, npts, generator=g), torch.randn(bs, nq, nh * hd, generator=g))
+    ref = oracle_all(inp)
+    d = to_device(inp, gpu_device)
+    gv = torch.empty_like(d.value)
+    gl, ga = _backward_c_abi(d, 2, gv)   # MXD_BWD_ANY_LAYOUT
+    keep = ~_cell_edge_mask(inp)[..., None]
+    assert rel_err(gv.double().cpu().numpy(), ref[1]) <= BWD_FP32
+    assert rel_err(gl.double().cpu().numpy() * keep, np.asarray(ref[2]) * keep) <= BWD_FP32
+    assert rel_err(ga.double().cpu().numpy(), ref[3]) <= BWD_FP32
