@@ -468,6 +468,12 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
         if (slices < 1.0) slices = 1.0;
         // (measured at the encoder shape: two slices side by side cost 10 to 15 % also where both fit the L2 --
         //  float16, 2 x 1.2 MB -- and 15 to 25 % where they do not -- float32, 2 x 2.4 MB)
+        // By default only where whole heads are pinned to an XCD, at most two of them: a head that several XCDs share
+        // needs so many workgroups per (batch, head) to keep the slices side by side on an XCD few that the cache fills
+        // outweigh the gain.  Measured at the encoder shape with the 16 (batch, head) pairs split as bs x heads --
+        // this form against the general kernel: 2 x 8: 91 / 102 us, 1 x 16: 96 / 123, 4 x 4: 102 / 102, 8 x 2: 120 / 105
+        // (152 with one round of workgroups), 16 x 1: 133 / 112 (175), 2 x 6 heads, no pinning: 106 / 94.
+        if (mode < 0 && (trial.xcd_mode != 1 || trial.heads_per_xcd > 2)) continue;
         double over = ceil(slices) * slice_bytes / (4.0 * 1024 * 1024) - 0.4;
         over = over < 0.0 ? 0.0 : (over > 1.0 ? 1.0 : over);
         const double gather = (1.0 + 0.5 * over) * (double)tq * (double)(d.nl * d.np) * 4.0;
@@ -477,6 +483,7 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
             best_p = P;
         }
     }
+    if (best_cost < 0.0) return false;  // (not a shape for this form)
     const int64_t tq = U * (((d.nq + best_p - 1) / best_p + U - 1) / U);
     const int64_t nt = (d.nq + tq - 1) / tq;
     memset(p, 0, sizeof(*p));
