@@ -101,6 +101,53 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
     return false;
 }
 
+// The samples of levels whose tiles found no room in the run table, added to grad_value one sample per thread with
+// atomics: share `part` of `parts` of the samples of (batch b, head h).  Only levels that overlap can have more tiles
+// between them than the table holds; for such layouts the whole image was zero-filled and every tile adds with atomics
+// as well.  Slow, and there so that level_start_index is honoured however it comes.  Plain operator only.
+// unfit: kMaxLevels flags in LDS, filled here.
+template <typename T>
+__device__ inline void add_levels_without_tiles(const KArgs& a, int b, int h, int part, int parts, int32_t* unfit)
+{
+    __shared__ int any_unfit;
+    if (threadIdx.x == 0) {
+        int32_t first = 0, any = 0;
+        for (int l = 0; l < a.nl; ++l) {
+            const i32x4 L = load_level(a, l);
+            int32_t P;
+            const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, &P);
+            const bool fits = first + nt <= a.tbl_stride - 1;
+            unfit[l] = fits ? 0 : 1;
+            if (fits) first += nt;
+            else if (nt > 0) any = 1;
+        }
+        any_unfit = any;
+    }
+    __syncthreads();
+    if (!any_unfit) return;
+    const T* loc = static_cast<const T*>(a.loc);
+    const T* attn = static_cast<const T*>(a.attn);
+    const T* gout = static_cast<const T*>(a.grad_out);
+    float* img = a.grad_value + (size_t)b * (a.gbatch_bytes / 4) + (size_t)h * a.hd;
+    const int64_t n = (int64_t)a.nq * a.S;
+    for (int64_t i = (int64_t)part * blockDim.x + threadIdx.x; i < n; i += (int64_t)parts * blockDim.x) {
+        const int q = (int)(i / a.S), s = (int)(i - (int64_t)q * a.S);
+        const int l = (int)(((uint32_t)s * a.np_magic) >> 20);
+        if (!unfit[l]) continue;
+        const int64_t e = (((int64_t)b * a.nq + q) * a.nh + h) * a.S_full + s;
+        const Sample sm = sample_geometry(to_f32(loc[2 * e]), to_f32(loc[2 * e + 1]), load_level(a, l), a.nk, true);
+        if (!sm.valid) continue;
+        const float aw = to_f32(attn[e]);
+        const T* grow = gout + (((int64_t)b * a.nq + q) * a.nh + h) * a.hd;
+        for (int ch = 0; ch < a.hd; ++ch) {
+            const float gch = to_f32(grow[ch]) * aw;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+                if (sm.cvalid[k]) unsafeAtomicAdd(img + (size_t)sm.pix[k] * ((size_t)a.nh * a.hd) + ch, sm.w[k] * gch);
+        }
+    }
+}
+
 // CH = channels a lane group accumulates per pass (registers); heads with more channels are
 // done in several passes over the same records.  VEC = elements per load of a grad_out row.
 template <typename T, int CH, int VEC>
@@ -138,6 +185,10 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         const int64_t r = (int64_t)wk.b * t.items_per_bh + wk.q_begin;
         wk.b = (int32_t)(r % a.bs);
         wk.q_begin = (int32_t)(r / a.bs);
+    }
+    if (wk.q_begin >= t.items_per_bh - t.extra) {  // (uniform: one of the workgroups behind the work items)
+        add_levels_without_tiles<T>(a, wk.b, wk.h, wk.q_begin - (t.items_per_bh - t.extra), t.extra, lv_first);
+        return;
     }
     if (threadIdx.x == 0) {
         item_ok = decode_tile_item(a, t, wk.q_begin, &item_s, lv_first, lv_nt) ? 1 : 0;

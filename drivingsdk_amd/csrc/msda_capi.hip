@@ -315,7 +315,7 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
 }
 
 // Geometry of the tile-ownership grad_value kernel (msda_bwd_tiles.hip).
-int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, mxd::TileArgs* t)
+int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, mxd::TileArgs* t, bool plain_operator = false)
 {
     memset(t, 0, sizeof(*t));
     // pair records (counted before merging) per work item when a hot tile is split: enough items to fill the 512
@@ -353,12 +353,14 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
     // work items per (batch, head): sum over levels of tiles*chunks <= 2*nl*nq*np/target + nl + sum of tiles
     const int64_t items = d.nl * ((2 * d.nq * d.np + t->target - 1) / t->target + 1) + L.tbl_stride;
     if (items >= (int64_t(1) << 24)) return fail(MXD_E_SHAPE, "backward needs %lld work items per (batch, head)", (long long)items);
-    t->items_per_bh = (int32_t)items;
+    t->items_per_bh = (int32_t)items;  // (the callers add TileArgs::extra)
     t->vec = vec;
     t->accumulate = accumulate;
     t->batch_major = tuning().tile_order > 0 ? 1 : 0;
     t->map.tile_q = 1;
-    const int64_t grid = fill_xcd_map(&t->map, d.bs, d.nh, items);
+    t->extra = plain_operator ? 8 : 0;
+    t->items_per_bh += t->extra;
+    const int64_t grid = fill_xcd_map(&t->map, d.bs, d.nh, t->items_per_bh);
     if (grid >= (int64_t(1) << 31)) return fail(MXD_E_SHAPE, "backward needs %lld workgroups, beyond the launch limit", (long long)grid);
     t->grid = (uint32_t)grid;
     t->block = mxd::kTilePx;
@@ -879,7 +881,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     const bool atomic_mode = !L.tiles || (flags & MXD_BWD_ANY_LAYOUT) != 0;
     mxd::TileArgs t;
     if (!atomic_mode) {
-        rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t);
+        rc = make_tile_args(d, L, a.plan.vec, (flags & MXD_BWD_ACCUMULATE) ? 1 : 0, &t, !fused && !gka && !grid);
         if (rc != MXD_OK) return rc;
         plan_image(&a, &t, half, (flags & MXD_BWD_ACCUMULATE) != 0, image, grad_value, hd);
     }

@@ -201,7 +201,9 @@ struct TileArgs {
     mxd_msda_plan map;     // only the XCD mapping fields are used: one "query" per work item
     int32_t target;        // pair records per work item aimed at when a hot tile is split by query range
     int32_t max_chunks;    // most query chunks a tile is split into
-    int32_t items_per_bh;  // upper bound of work items per (batch, head)
+    int32_t items_per_bh;  // upper bound of work items per (batch, head), including `extra`
+    int32_t extra;         // workgroups per (batch, head) behind the work items that add the samples of levels whose tiles
+                           // found no room in the run table (plain operator only; they leave at once otherwise)
     int32_t vec;           // elements per load of a grad_out row
     int32_t accumulate;    // add into the existing contents of the image
     int32_t store_vec;     // 4: rows of the image are 16-byte aligned, else 1

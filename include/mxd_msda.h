@@ -180,14 +180,15 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
 #define MXD_BWD_ACCUMULATE 1 /* fp32 only: add into the caller's grad_value instead of zero-filling it
                                 first (gradient accumulation; the caller owns the initial contents) */
 #define MXD_BWD_ANY_LAYOUT 2 /* take the one-kernel backward that adds to grad_value with global atomics (several
-                                times slower).  level_start_index is the caller's: the levels may leave keys uncovered
-                                and come in any order with every form of the backward; levels that OVERLAP are summed
-                                correctly by the default form only while they have no more than num_keys/512 +
-                                num_levels tiles of 512 pixels between them (always so when the level sizes add up to
-                                at most num_keys) -- beyond that the default form leaves a level out of grad_value,
-                                and this flag (or MXD_MSDA_BWD_ATOMIC=1 in the environment) is how to ask for the
-                                form that, like the reference's atomic-add kernel
-                                (op_kernel/multi_scale_deformable_attn_grad.cpp:181-186), does not care */
+                                times slower).  level_start_index is the caller's and is honoured as it comes by every
+                                form of the backward: the levels may leave keys uncovered, come in any order and
+                                overlap, as for the reference's atomic-add kernel
+                                (op_kernel/multi_scale_deformable_attn_grad.cpp:181-186).  One case is slow by default:
+                                levels that overlap so far that they have more than num_keys/512 + num_levels tiles of
+                                512 pixels between them -- mxd_msda_backward then adds the levels beyond that sample
+                                by sample.  The fused form and the sibling operators have no such fallback: there the
+                                default form leaves those levels out of grad_value, and this flag (or
+                                MXD_MSDA_BWD_ATOMIC=1 in the environment) asks for the form that does not care */
 
 /* Backward.  Replaces multi_scale_deformable_attn_backward
  * (mx_driving/csrc/MultiScaleDeformableAttn.cpp:68-118).  On `hip_stream`, in order:

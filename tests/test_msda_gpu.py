@@ -822,10 +822,12 @@ def test_level_start_indices_that_do_not_tile_the_keys(gpu_device, monkeypatch, 
     assert not np.any(got[1][:, ~covered]), "rows of grad_value outside every level must be exactly zero"
 
 
-def test_any_layout_flag_sums_levels_that_overlap_beyond_the_run_table(gpu_device):
+@pytest.mark.parametrize("flags", [0, 2], ids=["default", "MXD_BWD_ANY_LAYOUT"])
+def test_levels_that_overlap_beyond_the_run_table(gpu_device, flags):
     """Four levels that overlap so far that they have 17 tiles of 512 pixels between them while value has 3 422 keys
-    (room for 10 in the run table): with MXD_BWD_ANY_LAYOUT the backward takes the form with global atomics, which, like
-    the reference's kernel, takes level_start_index as it comes."""
+    (room for 10 in the run table).  By default the levels without room are added to grad_value sample by sample by
+    workgroups of the tile pass set aside for that; with MXD_BWD_ANY_LAYOUT the backward takes the one-kernel form with
+    global atomics.  Either way level_start_index is taken as it comes, as the reference's kernel takes it."""
     levels, starts, nk = ((56, 48), (10, 20), (58, 55), (58, 18)), (504, 1119, 148, 352), 3422
     bs, nq, nh, hd, npts = 2, 300, 4, 32, 5
     g = torch.Generator().manual_seed(77)
@@ -835,7 +837,7 @@ def test_any_layout_flag_sums_levels_that_overlap_beyond_the_run_table(gpu_devic
     ref = oracle_all(inp)
     d = to_device(inp, gpu_device)
     gv = torch.empty_like(d.value)
-    gl, ga = _backward_c_abi(d, 2, gv)   # MXD_BWD_ANY_LAYOUT
+    gl, ga = _backward_c_abi(d, flags, gv)
     keep = ~_cell_edge_mask(inp)[..., None]
     assert rel_err(gv.double().cpu().numpy(), ref[1]) <= BWD_FP32
     assert rel_err(gl.double().cpu().numpy() * keep, np.asarray(ref[2]) * keep) <= BWD_FP32
