@@ -86,6 +86,9 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     const int LPR = a.plan.lanes_per_row;
     const int lpr_log2 = __builtin_ctz(LPR);
     const int U = a.plan.units_per_wave;
+    // 2^sp neighbouring units share a query, each taking kChunk of its samples: a pass of a wavefront covers `span`
+    // samples of U >> sp queries (sp = 0: a unit is a query and goes through its samples kChunk at a time)
+    const int sp = a.unit_split_log2, sp_mask = (1 << sp) - 1, span = kChunk << sp;
     const int g = lane >> lpr_log2;
     const int c = lane & (LPR - 1);
     // lanes per row in the scatter phase: the power of two covering head_dim, within [LPR, 64]
@@ -130,7 +133,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     uint32_t gpk[NPASS][kPairs];
     auto unit_prologue = [&](int q0) {
         // grad_out row of this lane's unit in the value-load layout (for the dots)
-        const int qg = q0 + g;
+        const int qg = q0 + (g >> sp);
         const bool unit_ok = qg < wk.q_end;
         const T* grow = gout + (((int64_t)wk.b * a.nq + (unit_ok ? qg : wk.q_begin)) * a.nh + wk.h) * a.hd;
 #pragma unroll
@@ -170,7 +173,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             if (c == 0 && g < U) unit_stats(g)[2] = dsum;
             // softmax statistics: lanes 16u..16u+15 share unit u, each takes every 16th logit
             for (int i = lane; i < entries; i += kWave) {
-                const int u = i >> 4, sl = i & (kChunk - 1), q = q0 + u;
+                const int u = i >> 4, sl = i & (kChunk - 1), q = q0 + (u >> sp);
                 const T* lg = attn + (((int64_t)wk.b * a.nq + (q < wk.q_end ? q : wk.q_begin)) * a.nh + wk.h) * a.S_full;
                 float m = -__builtin_inff();
                 for (int s = sl; s < a.S; s += kChunk) m = __builtin_fmaxf(m, to_f32(lg[s]));
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         auto read_sample = [&](int i) -> Read {
             Read r{0.f, 0.f, 0.f, 0, false};
             const int u = i >> 4, sl = i & (kChunk - 1);
-            const int s = c0 + sl, q = q0 + u;
+            const int s = c0 + ((u & sp_mask) << 4) + sl, q = q0 + (u >> sp);
             r.active = (i < entries) && (q < wk.q_end) && (s < a.S);
             if (r.active) {
                 const SampleRef sr = sample_ref<SRC>(a, wk.b, q, wk.h, s);
@@ -304,9 +307,10 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         }
         for (int i = threadIdx.x; i < a.tbl_stride; i += blockDim.x) cursor[i] = 0;
         __syncthreads();
-        const int early_units = kEarly ? a.plan.waves_per_block * U : 0;  // their first kChunk samples are counted here:
+        // queries whose first `span` samples are counted here:
+        const int early_units = kEarly ? (a.plan.waves_per_block * U) >> sp : 0;
         if constexpr (kEarly) {
-            const int q0 = wk.q_begin + wave * U;
+            const int q0 = wk.q_begin + ((wave * U) >> sp);
             if (q0 < wk.q_end) {
                 if constexpr (FUSED) unit_prologue(q0);  // (the weights need the softmax terms)
                 geometry(q0, 0, std::true_type{});
@@ -317,11 +321,11 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         // the workgroup goes through every trip (the lane exchanges need their partners).
         const int S4 = (a.S + 3) & ~3;
         const int n = (wk.q_end - wk.q_begin) * S4;
-        const bool all_early = early_units >= wk.q_end - wk.q_begin && a.S <= kChunk;  // nothing left to count
+        const bool all_early = early_units >= wk.q_end - wk.q_begin && a.S <= span;  // nothing left to count
         for (int base = 0; base < n && !all_early; base += blockDim.x) {
             const int i = base + (int)threadIdx.x;
             const int qr = i / S4, s = i - qr * S4;
-            const bool act = i < n && s < a.S && !(qr < early_units && s < kChunk);
+            const bool act = i < n && s < a.S && !(qr < early_units && s < span);
             int l = 0;
             Sample sm;
             sm.cvalid[0] = sm.cvalid[1] = sm.cvalid[2] = sm.cvalid[3] = false;
@@ -384,7 +388,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     // wavefront has gathered, the staged entries are free, and a unit's 32 records (two per sample) fit the 16 entries
     // before its pad entry (which the fused form still needs).  Record `pos` of the slab lives at record pos % 32 of
     // unit pos / 32 of the workgroup.
-    const bool rec_in_lds = (SRC == kSrcPlain || SRC == kSrcFused) && !SCATTER && a.plan.iters == 1 && a.S <= kChunk;
+    const bool rec_in_lds = (SRC == kSrcPlain || SRC == kSrcFused) && !SCATTER && a.plan.iters == 1 && a.S <= span;
     const int u_log2 = __builtin_ctz(U);
     auto rec_lds = [&](int pos) {
         const int unit = pos >> 5;  // of the workgroup: wavefront unit >> u_log2, its unit & (U - 1)
@@ -406,7 +410,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     };
 
     for (int it = 0; it < a.plan.iters; ++it) {
-        const int q0 = wk.q_begin + (it * a.plan.waves_per_block + wave) * U;
+        const int q0 = wk.q_begin + (((it * a.plan.waves_per_block + wave) * U) >> sp);
         if (q0 >= wk.q_end) {
             if (rec_in_lds) {  // meets the other wavefronts at their two barriers and helps with the copy
                 __syncthreads();
@@ -418,7 +422,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 
         if (!(kEarly && FUSED && it == 0)) unit_prologue(q0);  // (the fused form's first iteration: done before the count)
 
-        for (int c0 = 0; c0 < a.S; c0 += kChunk) {
+        for (int c0 = 0; c0 < a.S; c0 += span) {
             // ---- geometry (the first chunk of the first iteration was staged while records were counted) ----
             if (!(kEarly && it == 0 && c0 == 0)) geometry(q0, c0, std::false_type{});
             wave_lds_sync();
@@ -477,7 +481,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 const int nsub = kWave >> span_log2;
                 const int sub = lane >> span_log2, ch0 = lane & ((1 << span_log2) - 1);
                 for (int u = sub; u < U; u += nsub) {
-                    const int qq = q0 + u;
+                    const int qq = q0 + (u >> sp);
                     if (qq >= wk.q_end) break;  // later units of this lane are past the end too
                     const T* gr = gout + (((int64_t)wk.b * a.nq + qq) * a.nh + wk.h) * a.hd;
                     const Entry* ent = stage + u * kChunkStride;
@@ -505,7 +509,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 const int i = lane + ks * kWave;
                 if (i >= entries) break;
                 const int u = i >> 4, sl = i & (kChunk - 1);
-                const int s = c0 + sl, q = q0 + u;
+                const int s = c0 + ((u & sp_mask) << 4) + sl, q = q0 + (u >> sp);
                 // the sample's pair records (upper and lower corners), written after the gradients
                 bool rec_have[2] = {false, false};
                 int32_t rec_key[2] = {0, 0};
@@ -671,7 +675,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         // slots of levels that attention_weights carries beyond spatial_shapes: zero gradients
         const int extra = a.S_full - a.S;
         if (extra > 0) {
-            for (int i = lane; i < U * extra; i += kWave) {
+            for (int i = lane; i < (U >> sp) * extra; i += kWave) {
                 const int u = i / extra, s = a.S + i % extra, q = q0 + u;
                 if (q < wk.q_end) {
                     const int64_t e = (((int64_t)wk.b * a.nq + q) * a.nh + wk.h) * a.S_full + s;

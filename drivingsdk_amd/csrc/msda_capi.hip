@@ -82,6 +82,7 @@ struct Tuning {
     int tile_order;      // MXD_MSDA_TILE_ORDER: 1 = work items of the tile pass batch-major, 0 = item-major, -1 = chosen here
     int bwd_sparse;      // MXD_MSDA_BWD_SPARSE: 0 = zero-fill (and, for 16-bit dtypes, round) the whole fp32 image of
                          // grad_value, 1 = only the rows that receive atomic additions
+    int bwd_unit_split;  // MXD_MSDA_BWD_UNIT_SPLIT: 0 = a unit of the first backward kernel is always a whole query
     int bwd_lane_bytes;  // MXD_MSDA_BWD_LANE_BYTES: most bytes of a row one lane of the first backward kernel loads
                          // (16, 8, 4), 0 = chosen here
 };
@@ -105,6 +106,7 @@ void read_tuning()
     t.tile_order = env_int("MXD_MSDA_TILE_ORDER", -1);
     t.bwd_lane_bytes = env_int("MXD_MSDA_BWD_LANE_BYTES", 0);
     t.bwd_sparse = env_int("MXD_MSDA_BWD_SPARSE", 1);
+    t.bwd_unit_split = env_int("MXD_MSDA_BWD_UNIT_SPLIT", 1);
     g_tuning = t;
 }
 
@@ -273,6 +275,13 @@ static int64_t bwd_tile_q(int dtype, const Dims& d)
     while (first > least && first * d.nl * d.np > samples) first >>= 1;
     for (int64_t tq = first; tq > least; tq >>= 1)
         if (d.bs * d.nh * ((d.nq + tq - 1) / tq) >= 6 * 256) return tq;
+    // Queries of 17 to 32 samples in a workgroup that makes one pass: two neighbouring units share a query, each taking
+    // 16 of its samples, so that the workgroup -- half as many queries -- stages all its samples while it counts its
+    // records (their geometry is derived once) and collects its records in LDS to write its slab in whole lines, as
+    // with up to 16 samples per query.
+    const int units = mxd::kWave / lpr * 4;
+    if (tuning().bwd_unit_split && least == units && units >= 8 && d.nl * d.np > mxd::kChunk && d.nl * d.np <= 2 * mxd::kChunk)
+        return least / 2;
     return least;
 }
 struct BwdLayout {
@@ -530,7 +539,14 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     if (iters < 1) iters = 1;
     const BwdLayout L = bwd_layout(dtype, d);
     // the tile pass wants L.tile_q queries per workgroup of the first backward kernel
-    if (backward) iters = L.tiles ? (int)(L.tile_q / (p->units_per_wave * p->waves_per_block)) : 1;
+    int split = 1;  // units of the backward's first kernel that share a query
+    if (backward) {
+        iters = L.tiles ? (int)(L.tile_q / (p->units_per_wave * p->waves_per_block)) : 1;
+        if (iters < 1) {
+            iters = 1;
+            split = (int)(p->units_per_wave * p->waves_per_block / L.tile_q);
+        }
+    }
     int cache = (level_cache && *level_cache && !backward) ? forward_cache_bytes(vec, es, d, p->units_per_wave) : 0;
     if (cache > 0) {
         // 8 wavefronts share one copy of the cached rows and work through 128 queries (MXD_MSDA_FWD_WGQ; 256 and
@@ -549,7 +565,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
         }
     }
     p->iters = iters;
-    p->tile_q = p->units_per_wave * p->waves_per_block * p->iters;
+    p->tile_q = p->units_per_wave * p->waves_per_block * p->iters / split;
     const int64_t ntiles = (d.nq + p->tile_q - 1) / p->tile_q;
     p->ntiles = (int32_t)ntiles;
     const int64_t grid = fill_xcd_map(p, d.bs, d.nh, ntiles);
@@ -574,6 +590,15 @@ int ptr_align(const void* p)
     int a = 16;
     while (a > 1 && (v & (uintptr_t)(a - 1))) a >>= 1;
     return a;
+}
+
+// Units of the backward's first kernel that share a query, as a power of two (see bwd_tile_q).
+int unit_split_log2(const mxd_msda_plan& p)
+{
+    const int units = p.units_per_wave * p.waves_per_block * p.iters;
+    int s = 0;
+    while (p.tile_q > 0 && (p.tile_q << (s + 1)) <= units) ++s;
+    return s;
 }
 
 void fill_args(mxd::KArgs* a, int dtype, const Dims& d)
@@ -846,6 +871,7 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     rc = make_plan(1, dtype, d, align, &a.plan);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.unit_split_log2 = unit_split_log2(a.plan);
     a.meta_i64 = meta64;
     a.value = value;
     a.shapes = spatial_shapes;
@@ -1084,6 +1110,7 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     rc = make_plan(1, dtype, d, align, &a.plan);
     if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.unit_split_log2 = unit_split_log2(a.plan);
     a.meta_i64 = meta64;
     fill_dagg(&a, num_cams, num_scale);
     a.value = mc_ms_feat;

@@ -72,6 +72,9 @@ struct KArgs {
     int32_t sparse;        // 1: only the rows of the image that receive atomic additions are zero-filled (and, for 16-bit
                            // dtypes, rounded afterwards): the other rows are stored once by the tile's owner
     void* grad_value_t;    // 16-bit dtypes with sparse = 1: the caller's grad_value, which receives those stores
+    int32_t unit_split_log2;  // backward's first kernel: 2^this units of a wavefront share a query, each taking kChunk of
+                           // its samples (unit u: query u >> this, samples ((u & (2^this - 1)) * kChunk ...); then
+                           // plan.tile_q = units per workgroup >> this
     int32_t bs, nk, nh, hd, nl, np, nq;
     int32_t S;             // nl*np: samples per unit that are evaluated
     int32_t S_full;        // nl_attn*np: samples per unit that are stored

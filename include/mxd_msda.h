@@ -81,7 +81,8 @@ typedef struct mxd_msda_plan {
     int32_t units_per_wave;  /* (query, head) units a wavefront handles side by side    */
     int32_t waves_per_block;
     int32_t iters;           /* wave-steps each wavefront runs                          */
-    int32_t tile_q;          /* queries per workgroup = units_per_wave*waves*iters      */
+    int32_t tile_q;          /* queries per workgroup = units_per_wave*waves*iters (half of that where the
+                                backward gives a query of 17 to 32 samples two units, 16 samples each) */
     int32_t ntiles;          /* query tiles per (batch, head)                           */
     int32_t xcd_mode;        /* 0 plain; 1 nh % 8 == 0 (heads pinned to an XCD);
                                 2 8 % nh == 0 (several XCDs share a head)               */
