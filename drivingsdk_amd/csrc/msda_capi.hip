@@ -437,10 +437,18 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
     const int cap = mxd::kCuLdsBytes - mxd::kCuTableBytes;  // (two level tables come first)
     const int64_t cap_rows = cap / (d.hd * es) - 1;
     const int64_t cached = estimated_cached_rows(d, cap_rows);
-    // By default (measured on MI355X): the form wins where about half of the samples are gathered from LDS and a unit's
-    // samples are one chunk -- the Deformable-DETR encoder shape, 84 against 97 us in float32 and 72 against 88 us in
-    // float16 -- and does not where a quarter are or a unit takes two chunks (BEVFormer's eight points per level:
-    // float32 389 against 420 us, float16 346 against 278 us; head_dim 128: equal), where the general kernel stays.
+    // By default (measured on MI355X, uniformly random locations, this form against the general kernel, float32 /
+    // float16).  Units of up to 16 samples (one chunk): it wins where about half of the samples are gathered from LDS
+    // -- the Deformable-DETR encoder shape, 79 against 86 us / 71 against 86 us; one level of 64 x 64 with 8 points,
+    // 85 against 106 / 77 against 97 -- and is level or behind where fewer are (BEVFormer's levels with 4 points: 214
+    // against 215 / 149 against 151; five levels: 258 against 206 / 185 against 179).  Units of more samples: it wins
+    // as soon as the last level is cached -- the encoder's levels with 5, 6, 8, 12, 16 points: 0.93, 0.91, 0.79, 0.76,
+    // 0.73 of the general kernel's time / 0.82, 0.78, 0.74, 0.68, 0.70; the BEVFormer shape 395 against 433 / 237
+    // against 288 -- unless a (batch, head) slice of value is far beyond an XCD's 4 MiB of L2, where the general
+    // kernel's larger number of wavefronts hides more of the memory latency (pyramid from 256 x 256, 11 MB in
+    // float32: 1750 against 1504 us; 5.6 MB in float16: 1109 against 1147; five levels from 200 x 300, 10 MB: 441
+    // against 404 / 5 MB: 287 against 308), and not where nothing is cached (one level of 100 x 150, 32 points: 153
+    // against 147 / 174 against 138).  Small problems stay with the general kernel (8 x 900 queries: 59 against 37).
     if (mode < 0) {
         double last = (double)d.nk, rows = 0.0;
         if (d.nl > 1) last = (double)d.nk * 3.0 / ((double)(int64_t(1) << (2 * (d.nl < 16 ? d.nl : 16))) - 1.0);
@@ -449,9 +457,8 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
             rows += r;
             ++levels_cached;
         }
-        if (2 * levels_cached < d.nl || d.nl * d.np > mxd::kChunk ||
-            d.bs * d.nh * d.nq * d.nl * d.np < (int64_t(1) << 20))
-            return false;
+        if (levels_cached == 0 || d.bs * d.nh * d.nq * d.nl * d.np < (int64_t(1) << 20)) return false;
+        if (d.nl * d.np <= mxd::kChunk ? 2 * levels_cached < d.nl : d.nk * d.hd * es > (int64_t(8) << 20)) return false;
     }
     const int U = mxd::kWave / lpr;
     const int64_t groups = (d.nq + U - 1) / U;
