@@ -458,7 +458,12 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
             ++levels_cached;
         }
         if (levels_cached == 0 || d.bs * d.nh * d.nq * d.nl * d.np < (int64_t(1) << 20)) return false;
-        if (d.nl * d.np <= mxd::kChunk ? 2 * levels_cached < d.nl : d.nk * d.hd * es > (int64_t(8) << 20)) return false;
+        const int64_t slice = d.nk * d.hd * es;
+        // (rows of 256 bytes, 16 samples per unit, one level of four cached: 0.88 to 0.93 of the general kernel's time at
+        //  the encoder's levels -- head_dim 64 and 48 in float32, 128 and 96 in float16, slices of 5 MB -- but 1.18 to
+        //  1.33 at slices of 8 MB and more, and 0.93 to 1.25 with 8 samples per unit)
+        const bool long_rows = lpr == 16 && d.nl * d.np == mxd::kChunk && slice <= (int64_t(6) << 20);
+        if (d.nl * d.np <= mxd::kChunk ? 2 * levels_cached < d.nl && !long_rows : slice > (int64_t(8) << 20)) return false;
     }
     const int U = mxd::kWave / lpr;
     const int64_t groups = (d.nq + U - 1) / U;
