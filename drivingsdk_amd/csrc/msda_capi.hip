@@ -801,8 +801,22 @@ int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, con
     if (ptr_align(output) < align) align = ptr_align(output);
     mxd::KArgs a;
     memset(&a, 0, sizeof(a));
-    rc = make_plan(0, dtype, d, align, &a.plan);
+    rc = ensure_device_ready();
     if (rc != MXD_OK) return rc;
+    // The one-workgroup-per-CU form takes reference points (x, y) and units of one chunk (the softmax is formed by the
+    // unit's lanes from the logits they hold); it reads offset pairs and reference points with one load each.
+    int cache = 0, cu = ref_dim == 2 && nl * np <= mxd::kChunk && ptr_align(sampling_offsets) >= 2 * elem_size(dtype) &&
+                        ptr_align(reference_points) >= 2 * elem_size(dtype);
+    if (cu) {
+        cache = 1;
+        rc = make_plan(0, dtype, d, align, &a.plan, &cache, &cu);
+        if (rc != MXD_OK) return rc;
+    }
+    if (!cu) {
+        cache = 0;
+        rc = make_plan(0, dtype, d, align, &a.plan);
+        if (rc != MXD_OK) return rc;
+    }
     fill_args(&a, dtype, d);
     a.meta_i64 = meta64;
     a.value = value;
@@ -813,7 +827,9 @@ int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, con
     a.ref = reference_points;
     a.ref_dim = ref_dim;
     a.out = output;
-    const hipError_t e = mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
+    a.lds_cache_bytes = cache;
+    const hipError_t e = cu ? mxd::launch_forward_cu(dtype, a, static_cast<hipStream_t>(hip_stream))
+                            : mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_fused_forward: launch failed: %s", hipGetErrorString(e));
     return MXD_OK;
 }

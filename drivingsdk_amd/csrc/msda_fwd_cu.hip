@@ -157,11 +157,17 @@ __device__ inline __amdgpu_buffer_rsrc_t vres_touch(const KArgs& a, const Work& 
 
 }  // namespace
 
-template <typename T, int VEC, int LPR>
+// SRC = kSrcFused: `loc` holds sampling offsets, `attn` logits and `ref` reference points (x, y) per (query, level);
+// location = reference + offset / (W, H), weight = softmax over the unit's samples (one chunk), formed by the unit's
+// lanes from the values they hold, with the arithmetic of the general kernel's fused form.
+template <typename T, int VEC, int LPR, int SRC>
 __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
 {
     static_assert(VEC * sizeof(T) == 16, "a lane owns 16 bytes of a row");
     static_assert(LPR == 4 || LPR == 8 || LPR == 16, "a unit lies inside a DPP row");
+    static_assert(SRC == kSrcPlain || SRC == kSrcFused, "the plain operator and its fused form");
+    constexpr bool FUSED = SRC == kSrcFused;
+    constexpr int LPR_LOG2 = LPR == 4 ? 2 : LPR == 8 ? 3 : 4;
     constexpr int U = kWave / LPR;     // units per wavefront
     constexpr int KS = kChunk / LPR;   // samples of a chunk per lane
     constexpr uint32_t ES = (uint32_t)sizeof(T);
@@ -284,6 +290,11 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
         make_rsrc(static_cast<const char*>(a.attn) + (size_t)wk.b * (loc_batch / 2), loc_batch / 2);
     const uint32_t out_batch = (uint32_t)a.nq * a.nh * row_bytes;
     const __amdgpu_buffer_rsrc_t ores = make_rsrc(static_cast<char*>(a.out) + (size_t)wk.b * out_batch, out_batch);
+    // fused form: reference points (x, y) of this batch element, one pair per (query, level)
+    const uint32_t ref_level_bytes = 2u * ES;
+    const uint32_t ref_batch = FUSED ? (uint32_t)a.nq * a.nl * ref_level_bytes : 0u;
+    const __amdgpu_buffer_rsrc_t rres =
+        make_rsrc(FUSED ? static_cast<const char*>(a.ref) + (size_t)wk.b * ref_batch : static_cast<const char*>(a.loc), ref_batch);
 
     // lanes past the end of the row read channel 0 and never store
     const bool chan_ok = c * VEC < a.hd;
@@ -301,16 +312,33 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
     const uint32_t loc_group_step = (uint32_t)q_step * a.nh * unit_loc_bytes;
     uint32_t out_off = ((uint32_t)q_lane * a.nh + wk.h) * row_bytes + lds_choff;
     const uint32_t out_group_step = (uint32_t)q_step * a.nh * row_bytes;
+    uint32_t ref_off = (uint32_t)q_lane * a.nl * ref_level_bytes;  // reference points of this lane's unit
+    const uint32_t ref_group_step = (uint32_t)q_step * a.nl * ref_level_bytes;
 
     // What this lane reads for chunk `ch` of its unit: the location and the weight of its KS samples of the chunk
     // (locations of the unit at byte offset `lo` of the batch element).  16-bit pairs and weights stay packed.
     struct Raw {
         uint32_t x, y, aw;  // float32: bit patterns; 16-bit types: x = the (x, y) pair, aw = the weight in the low half
+        uint32_t rx, ry;    // fused form: the reference point of the sample's level, laid out like (x, y)
     };
-    auto fetch = [&](uint32_t lo, int ch, Raw (&r)[KS]) {
+    auto fetch = [&](uint32_t lo, uint32_t ro, int ch, Raw (&r)[KS]) {
 #pragma unroll
         for (int k = 0; k < KS; ++k) {
             const uint32_t o = lo + (uint32_t)(ch * kChunk + k * LPR) * 2u * ES;
+            if constexpr (FUSED) {
+                const int s = ch * kChunk + k * LPR + c;
+                const int lraw = (int)(((uint32_t)s * a.np_magic) >> 20);
+                // (samples past the end of the list: any level's point, their weight is zero)
+                const uint32_t po = ro + (uint32_t)(lraw < a.nl ? lraw : 0) * ref_level_bytes;
+                if constexpr (sizeof(T) == 4) {
+                    const u32x2 p = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rres, po, 0, 0));
+                    r[k].rx = p.x;
+                    r[k].ry = p.y;
+                } else {
+                    r[k].rx = __builtin_bit_cast(uint32_t, __builtin_amdgcn_raw_buffer_load_b32(rres, po, 0, 0));
+                    r[k].ry = 0u;
+                }
+            }
             if constexpr (sizeof(T) == 4) {
                 const u32x2 xy = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(lres, o, 0, 0));
                 r[k].x = xy.x;
@@ -325,7 +353,7 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
     };
 
     Raw nxt[KS];
-    if (my_groups > 0) fetch(loc_off, 0, nxt);
+    if (my_groups > 0) fetch(loc_off, ref_off, 0, nxt);
     float acc[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
@@ -351,19 +379,42 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
                 // (samples past the end of the list take the empty level behind the last one: every corner outside)
                 const int lraw = (int)(((uint32_t)s * a.np_magic) >> 20);
                 const int l = lraw < a.nl ? lraw : a.nl;
-                float x, y, aw;
+                float x, y, aw, rx = 0.f, ry = 0.f;
                 if constexpr (sizeof(T) == 4) {
                     x = __builtin_bit_cast(float, nxt[K].x);
                     y = __builtin_bit_cast(float, nxt[K].y);
                     aw = __builtin_bit_cast(float, nxt[K].aw);
+                    if constexpr (FUSED) {
+                        rx = __builtin_bit_cast(float, nxt[K].rx);
+                        ry = __builtin_bit_cast(float, nxt[K].ry);
+                    }
                 } else {
                     typedef T t2 __attribute__((ext_vector_type(2)));
                     const t2 xy = __builtin_bit_cast(t2, nxt[K].x);
                     x = to_f32<T>(xy[0]);
                     y = to_f32<T>(xy[1]);
-                    aw = to_f32<T>(__builtin_bit_cast(T, (uint16_t)nxt[K].aw));
+                    // (the fused form's weights are float32 by now: see the softmax below)
+                    if constexpr (FUSED) aw = __builtin_bit_cast(float, nxt[K].aw);
+                    else aw = to_f32<T>(__builtin_bit_cast(T, (uint16_t)nxt[K].aw));
+                    if constexpr (FUSED) {
+                        const t2 rp = __builtin_bit_cast(t2, nxt[K].rx);
+                        rx = to_f32<T>(rp[0]);
+                        ry = to_f32<T>(rp[1]);
+                    }
                 }
-                cu_geometry(x, y, aw, active, tab.shape[l], tab.place[l], off, wgt);
+                const i32x4 shape = tab.shape[l];
+                if constexpr (FUSED) {
+                    // location = reference + offset / (W, H): every operation rounded on its own, as fused_location() does
+                    // (the backward derives the same locations and must land on the same pixels)
+#pragma clang fp contract(off)
+                    // (a bit cast applied directly to a vector element picks up element 0: copy first)
+                    const int32_t hb = shape.z, wb = shape.w;
+                    const float Hf = __builtin_bit_cast(float, hb), Wf = __builtin_bit_cast(float, wb);
+                    const float dx = x / Wf, dy = y / Hf;
+                    x = rx + dx;
+                    y = ry + dy;
+                }
+                cu_geometry(x, y, aw, active, shape, tab.place[l], off, wgt);
             };
             auto views = [&](auto g_c) {
                 constexpr int G = decltype(g_c)::value, K = (4 * G) / LPR, QO = ((4 * G) % LPR) / 4;
@@ -407,7 +458,7 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
             // workgroup's queries: nothing of it is used, and whatever lies beyond the tensor reads as zeros)
             auto fetch_next = [&]() {
                 const bool wrap = ch + 1 >= chunks;
-                fetch(wrap ? loc_off + loc_group_step : loc_off, wrap ? 0 : ch + 1, nxt);
+                fetch(wrap ? loc_off + loc_group_step : loc_off, wrap ? ref_off + ref_group_step : ref_off, wrap ? 0 : ch + 1, nxt);
             };
             constexpr int kLastGeometry = kChunk - LPR;  // the sample whose request computes the lane's last geometry
             // NM4 groups of four samples come from memory, the other 4 - NM4 from LDS
@@ -490,6 +541,30 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
                     samples_of(std::integral_constant<int, 3>{});
                 }
             };
+            if constexpr (FUSED) {
+                // softmax over the unit's samples (the launcher takes this form for units of one chunk only): every
+                // lane holds KS logits; maximum and sum of exponentials go round the unit's lanes with DPP, and the
+                // weights replace the logits as float32 bit patterns
+                float lg[KS], m = -__builtin_inff();
+                bool act[KS];
+#pragma unroll
+                for (int k = 0; k < KS; ++k) {
+                    act[k] = q_lane < wk.q_end && c0 + k * LPR + c < a.S;
+                    if constexpr (sizeof(T) == 4) lg[k] = __builtin_bit_cast(float, nxt[k].aw);
+                    else lg[k] = to_f32<T>(__builtin_bit_cast(T, (uint16_t)nxt[k].aw));
+                    if (act[k]) m = __builtin_fmaxf(m, lg[k]);
+                }
+                m = group_max<LPR_LOG2>(m);
+                float e[KS], sum = 0.0f;
+#pragma unroll
+                for (int k = 0; k < KS; ++k) {
+                    e[k] = act[k] ? expf(lg[k] - m) : 0.0f;
+                    sum += e[k];
+                }
+                sum = group_sum<LPR_LOG2>(sum);
+#pragma unroll
+                for (int k = 0; k < KS; ++k) nxt[k].aw = __builtin_bit_cast(uint32_t, act[k] ? e[k] / sum : 0.0f);
+            }
             int from_mem = s_cached - c0;  // samples of the chunk that come from memory
             from_mem = from_mem < 0 ? 0 : (from_mem > kChunk ? kChunk : from_mem);
             switch (from_mem) {
@@ -517,34 +592,35 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
         q_lane += q_step;
         loc_off += loc_group_step;
         out_off += out_group_step;
+        ref_off += ref_group_step;
     }
 }
 
-template <typename T>
+template <typename T, int SRC>
 static hipError_t launch_cu_t(const KArgs& a, hipStream_t stream)
 {
     constexpr int VEC = 16 / (int)sizeof(T);
     const dim3 grid(a.plan.grid), block(a.plan.block);
     switch (a.plan.lanes_per_row) {
-        case 4: hipLaunchKernelGGL((msda_fwd_cu_kernel<T, VEC, 4>), grid, block, a.plan.lds_bytes, stream, a); break;
-        case 8: hipLaunchKernelGGL((msda_fwd_cu_kernel<T, VEC, 8>), grid, block, a.plan.lds_bytes, stream, a); break;
-        case 16: hipLaunchKernelGGL((msda_fwd_cu_kernel<T, VEC, 16>), grid, block, a.plan.lds_bytes, stream, a); break;
+        case 4: hipLaunchKernelGGL((msda_fwd_cu_kernel<T, VEC, 4, SRC>), grid, block, a.plan.lds_bytes, stream, a); break;
+        case 8: hipLaunchKernelGGL((msda_fwd_cu_kernel<T, VEC, 8, SRC>), grid, block, a.plan.lds_bytes, stream, a); break;
+        case 16: hipLaunchKernelGGL((msda_fwd_cu_kernel<T, VEC, 16, SRC>), grid, block, a.plan.lds_bytes, stream, a); break;
         default: return hipErrorInvalidConfiguration;
     }
     return hipGetLastError();
 }
 
-template <typename T>
+template <typename T, int SRC>
 static hipError_t raise_lds_t()
 {
     constexpr int VEC = 16 / (int)sizeof(T);
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_cu_kernel<T, VEC, 4>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_cu_kernel<T, VEC, 4, SRC>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kCuLdsBytes);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_cu_kernel<T, VEC, 8>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_cu_kernel<T, VEC, 8, SRC>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kCuLdsBytes);
     if (e == hipSuccess)
-        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_cu_kernel<T, VEC, 16>),
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(&msda_fwd_cu_kernel<T, VEC, 16, SRC>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, kCuLdsBytes);
     return e;
 }
@@ -552,18 +628,23 @@ static hipError_t raise_lds_t()
 // Opt-in to more than 64 KiB of dynamic LDS for every instantiation, on the current device.
 hipError_t raise_forward_cu_lds()
 {
-    hipError_t e = raise_lds_t<float>();
-    if (e == hipSuccess) e = raise_lds_t<f16_t>();
-    if (e == hipSuccess) e = raise_lds_t<bf16_t>();
+    hipError_t e = raise_lds_t<float, kSrcPlain>();
+    if (e == hipSuccess) e = raise_lds_t<f16_t, kSrcPlain>();
+    if (e == hipSuccess) e = raise_lds_t<bf16_t, kSrcPlain>();
+    if (e == hipSuccess) e = raise_lds_t<float, kSrcFused>();
+    if (e == hipSuccess) e = raise_lds_t<f16_t, kSrcFused>();
+    if (e == hipSuccess) e = raise_lds_t<bf16_t, kSrcFused>();
     return e;
 }
 
+// (the fused form when a.ref is set: reference points (x, y), units of one chunk)
 hipError_t launch_forward_cu(int dtype, const KArgs& a, hipStream_t stream)
 {
+    const bool fused = a.ref != nullptr;
     switch (dtype) {
-        case MXD_DTYPE_F32: return launch_cu_t<float>(a, stream);
-        case MXD_DTYPE_F16: return launch_cu_t<f16_t>(a, stream);
-        case MXD_DTYPE_BF16: return launch_cu_t<bf16_t>(a, stream);
+        case MXD_DTYPE_F32: return fused ? launch_cu_t<float, kSrcFused>(a, stream) : launch_cu_t<float, kSrcPlain>(a, stream);
+        case MXD_DTYPE_F16: return fused ? launch_cu_t<f16_t, kSrcFused>(a, stream) : launch_cu_t<f16_t, kSrcPlain>(a, stream);
+        case MXD_DTYPE_BF16: return fused ? launch_cu_t<bf16_t, kSrcFused>(a, stream) : launch_cu_t<bf16_t, kSrcPlain>(a, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -8,7 +8,7 @@ import drivingsdk_amd
 from drivingsdk_amd import _lib, workloads
 from drivingsdk_amd.ops import msda_fused
 from oracle import msda_oracle as orc
-from util import BWD_FP32, FWD_FP32, HALF, rel_err
+from util import BF16, BWD_FP32, FWD_FP32, HALF, rel_err, set_tuning
 
 pytestmark = pytest.mark.gpu
 
@@ -105,6 +105,38 @@ def test_fused_forward_16bit(gpu_device, dtype):
     # half-ulp is up to 2^-8 of the element itself, which for the largest element is all of this error measure
     tol = HALF if dtype == torch.float16 else 2.0 ** -8
     assert rel_err(out.double().cpu().numpy(), want.numpy()) <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hd,nl,npts,nq", [(32, 4, 4, 1237), (32, 3, 5, 640), (16, 2, 8, 333), (64, 4, 2, 1001),
+                                           (8, 1, 13, 517), (128, 4, 4, 259)])
+def test_fused_forward_one_workgroup_per_cu_form(gpu_device, monkeypatch, hd, nl, npts, nq, dtype):
+    """The fused forward in the form that large problems take (one workgroup per CU, coarse levels in LDS, the softmax
+    formed by the unit's lanes), forced on small problems: rows of 4, 8 and 16 lanes, sample counts that are not a
+    multiple of four (the sample-by-sample loop), a last group of queries that is partly filled.  Against the oracle,
+    and against the general kernel's fused form (same arithmetic but for the order of the softmax sum)."""
+    g = torch.Generator().manual_seed(1000 + hd + npts)
+    shapes, lsi = workloads.level_tensors(((23, 31), (12, 16), (6, 8), (3, 4))[:nl])
+    nk = int(shapes.prod(1).sum())
+    bs, nh = 2, 3
+    value = torch.randn(bs, nk, nh, hd, generator=g).to(dtype)
+    ref = torch.rand(bs, nq, nl, 2, generator=g).to(dtype)
+    off = (torch.randn(bs, nq, nh, nl, npts, 2, generator=g) * 2).to(dtype)
+    logits = (torch.randn(bs, nq, nh, nl * npts, generator=g) * 2).to(dtype)
+    want = orc.fused_fwd_bwd(value, shapes, ref, off, logits, loc_dtype=torch.float32)[0].numpy()
+    args = [t.to(gpu_device) for t in (value, shapes, lsi, ref, off, logits)]
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    outs = {}
+    for mode in ("1", "0"):
+        set_tuning(monkeypatch, MXD_MSDA_FWD_CU=mode)
+        outs[mode] = drivingsdk_amd.multi_scale_deformable_attn_fused(*args).double().cpu().numpy()
+    # (the plan of the plain operator with the same sizes says which lane layout the forced form runs with)
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU="1")
+    eligible = hd * value.element_size() <= 256   # (rows of at most 16 lanes of 16 bytes)
+    assert (_lib.make_plan(0, code, bs, nk, nh, hd, nl, nl, nq, npts).block == 1024) == eligible
+    tol = FWD_FP32 if dtype == torch.float32 else HALF if dtype == torch.float16 else BF16
+    assert rel_err(outs["1"], want) <= tol
+    assert rel_err(outs["1"], outs["0"]) <= (2e-6 if dtype == torch.float32 else tol)
 
 
 def test_fused_more_than_16_samples_per_unit_and_many_heads(gpu_device):
