@@ -51,23 +51,59 @@ struct TileItem {
                                  // levels tile the keys, so that no tile of another level holds the same rows)
 };
 
+// What a workgroup needs of every level, derived by one lane per level (LevelInfo::fill) so that the thread that looks up
+// the work item afterwards goes through LDS values only: the level loads and the divisions behind the chunk count
+// would otherwise be made one level after the other by that one thread, in front of everything the workgroup does.
+struct LevelInfo {
+    int32_t H[kMaxLevels], W[kMaxLevels], base[kMaxLevels];
+    int32_t px[kMaxLevels];      // pixels of the level inside the value tensor
+    int32_t nt[kMaxLevels];      // its tiles (before the run table's room is considered)
+    int32_t chunks[kMaxLevels];  // query chunks per tile
+    int32_t wpc[kMaxLevels];     // first-kernel workgroups per chunk
+    __device__ void fill(const KArgs& a, int l)
+    {
+        const i32x4 L = load_level(a, l);
+        int32_t P, w = 0;
+        const int32_t n = level_tile_count(L.x, L.y, L.z, a.nk, &P);
+        H[l] = L.x;
+        W[l] = L.y;
+        base[l] = L.z;
+        px[l] = P;
+        nt[l] = n;
+        chunks[l] = n > 0 ? level_tile_chunks(a, n, &w) : 0;
+        wpc[l] = w;
+    }
+    // levels_tile_the_keys() on the values held here
+    __device__ bool tile_the_keys(const KArgs& a) const
+    {
+        int64_t next = 0;
+        int32_t tiles = 0;
+        for (int l = 0; l < a.nl; ++l) {
+            if (H[l] <= 0 || W[l] <= 0 || (int64_t)base[l] != next) return false;
+            const int64_t p = (int64_t)H[l] * W[l];
+            next += p;
+            if (next > a.nk) return false;
+            tiles += (int32_t)((p + kTilePx - 1) >> kTilePxLog2);
+        }
+        return next == a.nk && tiles <= a.tbl_stride - 1;
+    }
+};
+
 // lv_first / lv_nt: scratch of kMaxLevels entries each (first tile and tile count per level).
-__device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32_t item, TileItem* out,
+__device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, const LevelInfo& lv, int32_t item, TileItem* out,
                                         int32_t* lv_first, int32_t* lv_nt)
 {
     // Tiles are numbered level by level as in the first kernel; a level that does not fit the run table
     // (only possible when the levels overlap) has no tiles.
     int32_t total = 0;
     for (int l = 0; l < a.nl; ++l) {
-        int32_t P;
-        const i32x4 L = load_level(a, l);
-        const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, &P);
+        const int32_t nt = lv.nt[l];
         const bool fits = total + nt <= a.tbl_stride - 1;
         lv_first[l] = total;
         lv_nt[l] = fits ? nt : 0;
         if (fits) total += nt;
     }
-    const bool canonical = levels_tile_the_keys(a);
+    const bool canonical = lv.tile_the_keys(a);
     // Items are numbered from the last level to the first: the coarse levels, whose tiles are
     // split into many long-running items, start first and the short items of the fine levels
     // fill the end of the launch.
@@ -75,18 +111,14 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, int32
     for (int l = a.nl - 1; l >= 0; --l) {
         const int32_t nt = lv_nt[l];
         if (nt == 0) continue;
-        const i32x4 L = load_level(a, l);
-        const int32_t H = L.x, W = L.y, base = L.z;
-        int32_t P;
-        level_tile_count(H, W, base, a.nk, &P);
-        int32_t wpc;  // first-kernel workgroups per chunk
-        const int32_t chunks = level_tile_chunks(a, nt, &wpc);
+        const int32_t base = lv.base[l], P = lv.px[l];
+        const int32_t wpc = lv.wpc[l], chunks = lv.chunks[l];
         const int32_t n = nt * chunks;
         if (item < first + n) {
             const int32_t ti = (item - first) / chunks, ci = (item - first) % chunks;
             out->level = l;
-            out->H = H;
-            out->W = W;
+            out->H = lv.H[l];
+            out->W = lv.W[l];
             out->base = base;
             out->p0 = base + ti * kTilePx;
             out->p1 = (out->p0 + kTilePx) < (base + P) ? (out->p0 + kTilePx) : (base + P);
@@ -190,15 +222,21 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         add_levels_without_tiles<T>(a, wk.b, wk.h, wk.q_begin - (t.items_per_bh - t.extra), t.extra, lv_first);
         return;
     }
+    // (the per-level values live in the entry storage, which is not written before the work item is known: the kernel's
+    //  static LDS is 450 bytes short of the 80 KiB that let two workgroups share a CU)
+    static_assert(sizeof(LevelInfo) <= sizeof(u32x4) * kTileEntCap, "the level values must fit one wavefront's entry storage");
+    LevelInfo& lv_info = *reinterpret_cast<LevelInfo*>(&ent[0]);
+    if ((int)threadIdx.x < a.nl) lv_info.fill(a, (int)threadIdx.x);
+    if (threadIdx.x < kTilePx / 2) slot_info[threadIdx.x] = 0;
+    // an empty list points at the dummy entry of the wavefront that owns the pixel
+    heads[threadIdx.x] = (threadIdx.x >> 6) * kTileEntCap + kDummyOfWave;
+    __syncthreads();
     if (threadIdx.x == 0) {
-        item_ok = decode_tile_item(a, t, wk.q_begin, &item_s, lv_first, lv_nt) ? 1 : 0;
+        item_ok = decode_tile_item(a, t, lv_info, wk.q_begin, &item_s, lv_first, lv_nt) ? 1 : 0;
         done_count = 0;
         spare_next = 0;
         round1_total = 0;
     }
-    if (threadIdx.x < kTilePx / 2) slot_info[threadIdx.x] = 0;
-    // an empty list points at the dummy entry of the wavefront that owns the pixel
-    heads[threadIdx.x] = (threadIdx.x >> 6) * kTileEntCap + kDummyOfWave;
     __syncthreads();
     if (!item_ok) return;  // uniform
     const TileItem it = item_s;

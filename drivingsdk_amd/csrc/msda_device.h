@@ -104,13 +104,22 @@ constexpr int kRowParts = 16;  // pieces a tile's rows are cut into for the zero
 __device__ inline int32_t level_tile_chunks(const KArgs& a, int32_t nt, int32_t* wpc)
 {
     // two pair records per sample, spread evenly over the tiles of the level
-    const int64_t expect = (2 * (int64_t)a.nq * a.np) / nt;
-    int64_t chunks = (expect + a.tile_target - 1) / a.tile_target;
+    // (32-bit divisions wherever the operands allow: a 64-bit one is some 150 instructions, and the workgroups of all
+    //  three backward kernels go through this before they start)
+    const uint64_t records = 2 * (uint64_t)a.nq * (uint64_t)a.np;
+    const uint64_t expect = records <= 0xFFFFFFFFull ? (uint64_t)((uint32_t)records / (uint32_t)nt) : records / (uint64_t)nt;
+    const uint32_t target = (uint32_t)a.tile_target;
+    // (more chunks than the limit are cut down to it: the quotient itself is not needed then)
+    uint32_t chunks;
+    if (expect >= (uint64_t)target * (uint32_t)a.tile_max_chunks) chunks = (uint32_t)a.tile_max_chunks;
+    else if (expect <= 0xFFFFFFFFull - target) chunks = ((uint32_t)expect + target - 1) / target;
+    else chunks = (uint32_t)((expect + target - 1) / target);
     if (chunks < 1) chunks = 1;
-    if (chunks > a.tile_max_chunks) chunks = a.tile_max_chunks;
-    if (chunks > a.nwg) chunks = a.nwg;
-    *wpc = (int32_t)((a.nwg + chunks - 1) / chunks);
-    return (int32_t)((a.nwg + *wpc - 1) / *wpc);
+    if (chunks > (uint32_t)a.tile_max_chunks) chunks = (uint32_t)a.tile_max_chunks;
+    if (chunks > (uint32_t)a.nwg) chunks = (uint32_t)a.nwg;
+    const uint32_t w = ((uint32_t)a.nwg + chunks - 1) / chunks;
+    *wpc = (int32_t)w;
+    return (int32_t)(((uint32_t)a.nwg + w - 1) / w);
 }
 
 // A tile of `npx` pixels whose rows its one workgroup of the tile pass stores directly: no other workgroup adds to
