@@ -726,8 +726,8 @@ __global__ __launch_bounds__(256) void msda_round_rows_kernel(const KArgs a)
         const f32x4* src = reinterpret_cast<const f32x4*>(a.grad_value);
         t4* dst = reinterpret_cast<t4*>(a.grad_value_t);
         for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
-            const f32x4 v = src[i];
-            dst[i] = t4{from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])};
+            const f32x4 v = __builtin_nontemporal_load(src + i);  // (read once, written once)
+            __builtin_nontemporal_store(t4{from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])}, dst + i);
         }
         return;
     }
@@ -738,8 +738,8 @@ __global__ __launch_bounds__(256) void msda_round_rows_kernel(const KArgs a)
     t4* dst = reinterpret_cast<t4*>(a.grad_value_t) + ((size_t)b * a.nk + r0) * row4;
     const uint32_t n4 = (uint32_t)(r1 - r0) * row4;
     for (uint32_t i = threadIdx.x; i < n4; i += blockDim.x) {
-        const f32x4 v = src[i];
-        dst[i] = t4{from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])};
+        const f32x4 v = __builtin_nontemporal_load(src + i);
+        __builtin_nontemporal_store(t4{from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])}, dst + i);
     }
 }
 
