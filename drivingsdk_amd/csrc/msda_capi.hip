@@ -334,7 +334,9 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
     // (0.17 M samples: 2 100, 0.5 M: 3 600, 1.3 M: 5 700 records per item).
     int64_t target = 2 * d.bs * d.nh * d.nq * d.nl * d.np / 512;
     if (target < 8192) target = (int64_t)sqrt(8192.0 * (double)(target > 32 ? target : 32));
-    if (target > 32768) target = 32768;
+    // (capped: 32 768 measured 0.6 to 1.7 % behind 49 152 on problems of 10 to 40 M samples, 65 536 up to 4 % behind it and
+    //  100 000 up to 20 %: the launch then has too few items to fill the chip evenly)
+    if (target > 49152) target = 49152;
     if (d.nl == 1) {
         // One level: its tiles all collect about the same number of records, so the launch is a whole number of
         // equal work items per tile.  Up to 512 of them run side by side in the chip's workgroup slots; a few more
