@@ -440,6 +440,14 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
     const int mode = tuning().fwd_cu;
     const int es = elem_size(dtype);
     if (mode == 0 || vec * es != 16 || npass != 1 || lpr > 16) return false;
+    // What the kernel's index arithmetic assumes, whatever the environment asks for: pixel indices and the distance
+    // between neighbouring pixels are multiplied as 24-bit integers, and the locations, weights, results (and the
+    // fused form's reference points) of one batch element are addressed with 32-bit byte offsets inside a buffer
+    // descriptor.  Anything larger goes to the general kernel, which indexes with 64-bit offsets.
+    const int64_t kMul24 = int64_t(1) << 23, kOff32 = int64_t(1) << 31;
+    if (d.nk >= kMul24 || d.nh * d.hd * es >= kMul24 || d.nq * d.nh * d.nl_attn * d.np * 2 * es >= kOff32 ||
+        d.nq * d.nh * d.hd * es >= kOff32 || d.nq * d.nl * 2 * es >= kOff32)
+        return false;
     const int cap = mxd::kCuLdsBytes - mxd::kCuTableBytes;  // (two level tables come first)
     const int64_t cap_rows = cap / (d.hd * es) - 1;
     const int64_t cached = estimated_cached_rows(d, cap_rows);

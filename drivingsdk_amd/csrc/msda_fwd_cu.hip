@@ -103,8 +103,8 @@ struct LevelTables {
 
 // Geometry of one sample: byte offsets of its four corner rows (the "outside" offset for corners that must not
 // be touched) and the bilinear weights times the attention weight, as bit patterns.  Same arithmetic and the same
-// order of operations as sample_geometry(); the pixel offset is formed with 24-bit multiplies (the launcher only
-// picks this kernel when pixel counts and strides are below 2^23).
+// order of operations as sample_geometry(); the pixel offset is formed with 24-bit multiplies (plan_forward_cu()
+// refuses this kernel unless the key count and the distance between neighbouring pixels are below 2^23).
 __device__ inline void cu_geometry(float x, float y, float aw, bool active, const i32x4 shape, const u32x4 place,
                                    uint32_t (&off)[4], uint32_t (&wgt)[4])
 {
@@ -282,7 +282,8 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
 
     const __amdgpu_buffer_rsrc_t vres =
         make_rsrc(static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes, a.batch_bytes);
-    // locations, weights and results of this batch element (the launcher checked that each stays below 2 GiB)
+    // locations, weights and results of this batch element (plan_forward_cu() refuses this kernel unless each -- and the
+    // fused form's reference points -- stays below 2 GiB, so that the 32-bit offsets below cannot wrap)
     const uint32_t unit_loc_bytes = (uint32_t)a.S_full * 2u * ES;  // locations of one (query, head)
     const uint32_t loc_batch = (uint32_t)a.nq * a.nh * unit_loc_bytes;
     const __amdgpu_buffer_rsrc_t lres = make_rsrc(static_cast<const char*>(a.loc) + (size_t)wk.b * loc_batch, loc_batch);

@@ -329,3 +329,37 @@ def test_backward_plans_stay_inside_the_default_lds_limit():
                     for nl in (1, 4):
                         plan = _lib.make_plan(1, dtype, 1, nk, nh, hd, nl, nl, 1000, 4)
                         assert plan.lds_bytes <= 64 * 1024, (dtype, hd, nh, nk, nl, plan.lds_bytes, es)
+
+
+@pytest.mark.parametrize("forced", [None, 1])
+def test_forward_cu_form_is_refused_beyond_its_index_arithmetic(monkeypatch, forced):
+    """The forward's one-workgroup-per-CU form multiplies pixel indices and pixel strides as 24-bit integers and
+    addresses the locations, weights and results of a batch element with 32-bit byte offsets: problems beyond that must
+    get the general kernel's plan (block != 1024), also when the environment forces the form on
+    (reference: the same class of overflow is flagged in kernels/multi_scale_deformable_attn/op_kernel/msda.h:428)."""
+    from util import set_tuning
+    if forced is not None:
+        set_tuning(monkeypatch, MXD_MSDA_FWD_CU=forced)
+    # bs, nk, nh, hd, nl, nl_attn, nq, np -- each just beyond one of the limits, all inside what a call accepts
+    beyond = [
+        (1, (1 << 23) + 1, 8, 4, 4, 4, 300_000, 4),          # key count: 24-bit pixel index
+        (2, 19947, 8, 32, 4, 4, 1 << 21, 4),                  # locations of a batch element: 2^21*8*16*8 B = 2 GiB
+        (2, 19947, 8, 32, 4, 4, (1 << 21) + 1, 1),            # results of a batch element: > 2 GiB
+    ]
+    for dtype in (0, 1, 2):
+        es = 4 if dtype == 0 else 2
+        for dims in beyond:
+            bs, nk, nh, hd, nl, nla, nq, npts = dims
+            if nk * nh * hd * 4 >= 1 << 31:
+                continue
+            plan = _lib.make_plan(0, dtype, *dims)
+            over_loc = nq * nh * nla * npts * 2 * es >= 1 << 31
+            over_out = nq * nh * hd * es >= 1 << 31
+            if nk >= 1 << 23 or over_loc or over_out:
+                assert plan.block != 1024, (dtype, dims, plan.as_dict())
+    # the form is still what the benchmark shape gets (forced or by default)
+    assert _lib.make_plan(0, 0, 2, 19947, 8, 32, 4, 4, 19947, 4).block == 1024
+    # distance between neighbouring pixels of 2^23 bytes and more (fp32, forced form): general kernel
+    if forced:
+        plan = _lib.make_plan(0, 0, 1, 60, 32768, 64, 1, 1, 1 << 16, 16)
+        assert plan.block != 1024, plan.as_dict()
