@@ -93,16 +93,23 @@ def _kernel_times(d, iters, warmup):
     # After an idle period the GPU's clocks rise over about the first 30 ms of back-to-back work (and fall back
     # within a few ms without work), which is longer than any of the timed loops below: run that long first, so
     # that every figure is of the state in which a training job runs.
-    t_end = time.perf_counter() + 0.05
+    t_begin = time.perf_counter()
+    t_end = t_begin + 0.05
+    lead_in_launches = 0
     while time.perf_counter() < t_end:
         for _ in range(25):
             bwd(0)
+        lead_in_launches += 25
         torch.cuda.synchronize()
+    lead_in_ms = (time.perf_counter() - t_begin) * 1e3
 
     plan = _lib.make_plan(0, code, *dims)
     res = {"forward_kernel": "msda_fwd_cu_kernel" if plan.block == 1024 else "msda_fwd_kernel",
            "forward_ms": _event_ms(fwd, iters, warmup), "backward_with_zero_fill_ms": _event_ms(lambda: bwd(0), iters, warmup)}
     n_single = min(max(iters, 20), 100)
+    # what ran on the GPU between the first call and the declared warm-up steps (see main())
+    res["lead_in"] = {"backward_launches": lead_in_launches, "ms": lead_in_ms,
+                      "timed_kernel_launches_after_it": 2 * (iters + warmup) + 2 * n_single + (iters + warmup if code == 0 else 0)}
     res["forward_single_launch_ms"] = _event_stats_ms(fwd, n_single)
     res["backward_single_launch_ms"] = _event_stats_ms(lambda: bwd(0), n_single)
     # rate at which the forward moves corner rows (4 per sample) from cache to the CUs
@@ -199,41 +206,40 @@ def _physical_cores():
         return None
 
 
-def _cpu_baseline(inp, max_seconds=16.0):
+def _cpu_baseline(inp, warmups=3, timed=5, max_seconds=60.0):
     """The CPU oracle (grid_sample formulation, float32, autograd backward) on the host cores: whole forward+backward
-    iterations of the same workload, as many as fit the time bound -- with the threads this process may use (torch's
-    default: the box's CPU share) and, for reference, with one thread."""
+    iterations of the same workload -- `warmups` untimed ones, then `timed` timed ones, median -- with the threads
+    this process may use (torch's default: the box's CPU share) and, for reference, with one thread.  A run that
+    passes `max_seconds` stops early, with at least one timed iteration, and says how many it made."""
     import torch
 
     from oracle import msda_oracle as orc
 
-    def run(threads, bound, most):
+    def run(threads):
         torch.set_num_threads(threads)
         times = []
         t_begin = time.perf_counter()
-        it = 0
-        while True:
+        for it in range(warmups + timed):
             t0 = time.perf_counter()
             orc.msda_grid_sample_fwd_bwd(inp.value, inp.spatial_shapes, inp.sampling_locations, inp.attention_weights,
                                          inp.grad_output, dtype=torch.float32)
             t1 = time.perf_counter()
-            if it > 0:  # first iteration is a warm-up
+            if it >= warmups:
                 times.append(t1 - t0)
-            it += 1
-            if len(times) >= most or ((time.perf_counter() - t_begin) > bound and times):
+            if times and (t1 - t_begin) > max_seconds:
                 break
         return statistics.median(times), len(times)
 
     threads = torch.get_num_threads()
     nqueries = inp.sampling_locations.shape[0] * inp.sampling_locations.shape[1]
-    med, n = run(threads, max_seconds, 5)
-    med1, n1 = run(1, max_seconds, 2)
+    med, n = run(threads)
+    med1, n1 = run(1)
     torch.set_num_threads(threads)
     return {"value": nqueries / med, "unit": "queries/s", "cores": threads, "kind": "port",
             "ms_per_step": med * 1e3, "host_physical_cores": _physical_cores(), "host_logical_cpus": os.cpu_count(),
             "single_thread": {"value": nqueries / med1, "unit": "queries/s", "cores": 1, "ms_per_step": med1 * 1e3,
-                              "sample": f"{n1} timed iteration(s) after 1 warm-up"},
-            "sample": f"{n} timed forward+backward iterations (median) of the full workload after 1 warm-up, "
+                              "sample": f"{n1} timed iterations (median) after {warmups} warm-ups"},
+            "sample": f"{n} timed forward+backward iterations (median) of the full workload after {warmups} warm-ups, "
                       f"torch grid_sample formulation in float32 with {threads} threads (the CPU share of a one-GPU box)"}
 
 
@@ -436,6 +442,8 @@ def main():
     ap.add_argument("--workload", default="detr_encoder_bwd")
     ap.add_argument("--dtype", default="float32", choices=["float32", "float16", "bfloat16"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-iters", default="3,5", metavar="WARMUPS,TIMED",
+                    help="iterations of the CPU baseline per thread count (default: 3 warm-ups, 5 timed, median)")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run a plain elementwise copy kernel of value's size (reads and writes "
                          "value.numel()*4 bytes) so that FETCH_SIZE/WRITE_SIZE of a rocprofv3 --pmc run "
@@ -484,6 +492,12 @@ def main():
     # spends its life past that rise. The kernel timings run that long before they time anything.
     step()
     torch.cuda.synchronize()
+    # the same K steps straight after that first call, i.e. at the start of the clock rise: the other clock state
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    cold_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     k = _kernel_times(d, iters=max(args.steps, 50), warmup=max(args.warmup, 10))
 
     for _ in range(args.warmup):
@@ -528,8 +542,14 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
-        "before_warmup": "one untimed step (first-call allocations), then the per-kernel event timings of 'kernels' "
-                         "(which start with 50 ms of back-to-back launches: the GPU's clocks take ~30 ms to rise)",
+        "cold_ms_per_step": cold_ms_per_step,
+        "before_warmup": "one untimed step (first-call allocations), the K steps of cold_ms_per_step (timed straight "
+                         "after it, inside the rise of the GPU's clocks), then the per-kernel event timings of 'kernels' "
+                         "(which start with 50 ms of back-to-back launches: the clocks take ~30 ms to rise); "
+                         "kernels.lead_in counts them",
+        "effective_warmup": {"steps_through_autograd": 1 + args.steps + args.warmup,
+                             "raw_kernel_launches": k["lead_in"]["backward_launches"] +
+                             k["lead_in"]["timed_kernel_launches_after_it"]},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -549,7 +569,8 @@ def main():
     if args.dtype == "float32":
         result["module_forward"] = _module_forward_times(d, iters=max(args.steps, 50), warmup=max(args.warmup, 10))
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = _cpu_baseline(inp)
+        cpu_warmups, cpu_timed = (int(x) for x in args.cpu_iters.split(","))
+        result["cpu_baseline"] = _cpu_baseline(inp, warmups=cpu_warmups, timed=max(cpu_timed, 1))
         result["speedup_vs_cpu_baseline"] = result["value"] / result["cpu_baseline"]["value"]
     print(json.dumps(result))
 

@@ -20,7 +20,8 @@ def _run(*args):
 
 
 def test_default_workload_line(gpu_device):
-    r = _run("--gpus", "1", "--steps", "5", "--warmup", "2")
+    # (the CPU baseline with one warm-up and one timed iteration per thread count: its keys are what is checked here)
+    r = _run("--gpus", "1", "--steps", "5", "--warmup", "2", "--cpu-iters", "1,1")
     assert r["metric"].startswith("MSDA fwd+bwd queries/s") and r["unit"] == "queries/s"
     assert r["n_gpus"] == 1 and r["steps"] == 5 and r["warmup"] == 2
     assert r["higher_is_better"] is True and r["scaling"] == "weak" and r["vs_baseline"] is None
@@ -28,7 +29,9 @@ def test_default_workload_line(gpu_device):
     assert r["config"]["workload"].startswith("detr_encoder_bwd") and "model" not in r["config"]
     queries = 2 * 19947
     assert abs(r["value"] - queries / (r["ms_per_step"] * 1e-3)) <= 1e-6 * r["value"]
-    assert 2e7 < r["value"] < 1e9
+    assert r["value"] > 0 and r["cold_ms_per_step"] > 0
+    assert r["effective_warmup"]["steps_through_autograd"] == 1 + 5 + 2
+    assert r["effective_warmup"]["raw_kernel_launches"] >= r["kernels"]["lead_in"]["backward_launches"] > 0
     for key in ("roofline", "roofline_forward", "roofline_backward"):
         f = r[key]
         assert f["bound"] == "hbm" and f["unit"] == "GB/s" and f["peak"] == 8000.0
@@ -41,8 +44,8 @@ def test_default_workload_line(gpu_device):
     assert r["roofline_backward"]["algorithmic_bytes"] == 6144 * queries
     c = r["cpu_baseline"]
     assert c["kind"] == "port" and c["unit"] == "queries/s" and c["cores"] >= 1 and c["value"] > 0 and c["sample"]
-    assert c["single_thread"]["cores"] == 1 and 0 < c["single_thread"]["value"] <= c["value"] * 1.5
-    assert r["value"] > 50 * c["value"]
+    assert c["single_thread"]["cores"] == 1 and c["single_thread"]["value"] > 0
+    assert abs(r["speedup_vs_cpu_baseline"] - r["value"] / c["value"]) <= 1e-6 * r["speedup_vs_cpu_baseline"]
 
 
 def test_other_workload_line_without_committed_traffic(gpu_device):
