@@ -39,6 +39,7 @@ struct KArgs {
     uint32_t sc_magic;     // ceil(2^20/scales): level / scales
     int32_t lds_cache_bytes;  // forward: LDS set aside for the rows of the last (coarsest) levels, 0 = none
     int32_t fwd_ahead;        // forward: request an iteration's samples before the gather of the one before it
+    int32_t fwd_cu_flip;      // forward, one workgroup per CU: half of the wavefronts take their LDS groups first
     int32_t grid_h, grid_w;  // grid sampler: the one level's shape comes with the call, not from device memory
     int32_t grid;          // grid sampler: 1 + padding mode (0 zeros, 1 border) + 2*align_corners; 0 = not a grid sampler
     int32_t gka;           // geometric kernel attention: locations are pixel indices, one pixel per sample

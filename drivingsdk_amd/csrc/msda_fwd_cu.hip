@@ -279,6 +279,9 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
     const int nwaves = blockDim.x >> 6;
     const int g = lane / LPR;  // unit slot of this lane
     const int c = lane % LPR;  // position inside the row
+    // wavefronts 4..7 and 12..15 of the workgroup (two of the four on every SIMD) work through their chunks from the LDS
+    // groups on (see `pipelined`)
+    const bool flipped = a.fwd_cu_flip != 0 && ((wave >> 2) & 1) != 0;
 
     const __amdgpu_buffer_rsrc_t vres =
         make_rsrc(static_cast<const char*>(a.value) + (size_t)wk.b * a.batch_bytes, a.batch_bytes);
@@ -426,24 +429,25 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
                     vw[G & 1][j] = unit_view<LPR, QO>(wgt[j]);
                 }
             };
-            auto load_sample = [&](auto i_c, auto lds_c) {
-                constexpr int I = decltype(i_c)::value, G = I / 4, J = I % 4;
+            // (I: the sample of the chunk; R: its place in the ring of rows)
+            auto load_sample = [&](auto i_c, auto r_c, auto lds_c) {
+                constexpr int I = decltype(i_c)::value, R = decltype(r_c)::value, G = I / 4, J = I % 4;
                 if constexpr (decltype(lds_c)::value) {
 #pragma unroll
                     for (int k = 0; k < 4; ++k)
-                        raw[I % kRing][k] = *reinterpret_cast<const raw_t*>(cache + (quad_bcast<J>(vo[G & 1][k]) + lds_choff));
+                        raw[R][k] = *reinterpret_cast<const raw_t*>(cache + (quad_bcast<J>(vo[G & 1][k]) + lds_choff));
                 } else {
 #pragma unroll
                     for (int k = 0; k < 4; ++k)
-                        raw[I % kRing][k] = RowIO<T, VEC>::load_raw(vres, quad_bcast<J>(vo[G & 1][k]) + choff);
+                        raw[R][k] = RowIO<T, VEC>::load_raw(vres, quad_bcast<J>(vo[G & 1][k]) + choff);
                 }
             };
-            auto use_sample = [&](auto i_c) {
-                constexpr int I = decltype(i_c)::value, G = I / 4, J = I % 4;
+            auto use_sample = [&](auto i_c, auto r_c) {
+                constexpr int I = decltype(i_c)::value, R = decltype(r_c)::value, G = I / 4, J = I % 4;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     float v[VEC];
-                    RowIO<T, VEC>::unpack(raw[I % kRing][k], v);
+                    RowIO<T, VEC>::unpack(raw[R][k], v);
                     if constexpr (sizeof(T) == 4) {
 #pragma unroll
                         for (int e = 0; e < VEC; ++e) fma_quad_bcast<J>(acc[e], vw[G & 1][k], v[e]);
@@ -462,22 +466,33 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
                 fetch(wrap ? loc_off + loc_group_step : loc_off, wrap ? ref_off + ref_group_step : ref_off, wrap ? 0 : ch + 1, nxt);
             };
             constexpr int kLastGeometry = kChunk - LPR;  // the sample whose request computes the lane's last geometry
-            // NM4 groups of four samples come from memory, the other 4 - NM4 from LDS
-            auto pipelined = [&](auto nm4_c) {
+            // NM4 groups of four samples come from memory, the other 4 - NM4 from LDS.  FLIP: the chunk is worked through
+            // from its first LDS group on, round to its memory groups (step P of the chunk takes sample (P + 4 NM4) mod
+            // 16).  Half of a CU's wavefronts run flipped, two on every SIMD, so that at any moment about half of them
+            // gather from memory -- the vector-memory pipeline is what they wait for -- while the other half gather
+            // from LDS and keep the vector ALU busy, instead of all sixteen meeting in front of the same unit phase
+            // after phase.  (The sum of a flipped wavefront's unit is formed in that order as well.)
+            auto pipelined = [&](auto nm4_c, auto flip_c) {
                 constexpr int NM4 = decltype(nm4_c)::value;
+                constexpr bool FLIP = decltype(flip_c)::value;
+                constexpr int kRot = FLIP ? 4 * NM4 : 0;  // the sample that step 0 takes
+                static_assert(kRot % LPR == 0, "a flipped chunk starts with the first group of a lane's sample");
                 constexpr int kLastMem = 4 * NM4 - 1;
-                constexpr int kFetchAfter = kLastMem > kLastGeometry ? kLastMem : kLastGeometry;  // after this sample's request
-                auto load = [&](auto i_c) {
-                    constexpr int I = decltype(i_c)::value;
+                // after this step's request (flipped: the memory groups end the chunk, and the next chunk's first
+                // geometry should not find its locations still on their way)
+                constexpr int kFetchAfter = FLIP ? kLastGeometry : (kLastMem > kLastGeometry ? kLastMem : kLastGeometry);
+                auto load = [&](auto p_c) {
+                    constexpr int P = decltype(p_c)::value, I = (P + kRot) % kChunk;
                     if constexpr (I % 4 == 0) views(std::integral_constant<int, I / 4>{});
-                    load_sample(i_c, std::integral_constant<bool, (I / 4 >= NM4)>{});
-                    if constexpr (I == kFetchAfter) fetch_next();
+                    load_sample(std::integral_constant<int, I>{}, std::integral_constant<int, P % kRing>{},
+                                std::integral_constant<bool, (I / 4 >= NM4)>{});
+                    if constexpr (P == kFetchAfter) fetch_next();
                 };
-                auto step = [&](auto i_c) {
-                    constexpr int I = decltype(i_c)::value;
-                    if constexpr (I + kRing - 1 < kChunk) load(std::integral_constant<int, I + kRing - 1>{});
+                auto step = [&](auto p_c) {
+                    constexpr int P = decltype(p_c)::value, I = (P + kRot) % kChunk;
+                    if constexpr (P + kRing - 1 < kChunk) load(std::integral_constant<int, P + kRing - 1>{});
                     __builtin_amdgcn_sched_barrier(0);  // requests go out before the rows of an earlier sample are waited for
-                    use_sample(i_c);
+                    use_sample(std::integral_constant<int, I>{}, std::integral_constant<int, P % kRing>{});
                     __builtin_amdgcn_sched_barrier(0);
                 };
                 load(std::integral_constant<int, 0>{});
@@ -568,12 +583,23 @@ __global__ __launch_bounds__(1024) void msda_fwd_cu_kernel(const KArgs a)
             }
             int from_mem = s_cached - c0;  // samples of the chunk that come from memory
             from_mem = from_mem < 0 ? 0 : (from_mem > kChunk ? kChunk : from_mem);
+            // (a chunk can be flipped when its first LDS group is the first group of a lane's sample)
+            auto either = [&](auto nm4_c) {
+                constexpr int NM4 = decltype(nm4_c)::value;
+                if constexpr ((4 * NM4) % LPR == 0 && NM4 > 0 && NM4 < 4) {
+                    if (flipped) {
+                        pipelined(nm4_c, std::true_type{});
+                        return;
+                    }
+                }
+                pipelined(nm4_c, std::false_type{});
+            };
             switch (from_mem) {
-                case 0: pipelined(std::integral_constant<int, 0>{}); break;
-                case 4: pipelined(std::integral_constant<int, 1>{}); break;
-                case 8: pipelined(std::integral_constant<int, 2>{}); break;
-                case 12: pipelined(std::integral_constant<int, 3>{}); break;
-                case 16: pipelined(std::integral_constant<int, 4>{}); break;
+                case 0: either(std::integral_constant<int, 0>{}); break;
+                case 4: either(std::integral_constant<int, 1>{}); break;
+                case 8: either(std::integral_constant<int, 2>{}); break;
+                case 12: either(std::integral_constant<int, 3>{}); break;
+                case 16: either(std::integral_constant<int, 4>{}); break;
                 default: serial(); break;
             }
         }
