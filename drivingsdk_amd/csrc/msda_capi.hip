@@ -79,7 +79,8 @@ struct Tuning {
                          // -1 = for problems large enough to pay for it
     int fwd_cu_wgs;      // MXD_MSDA_FWD_CU_WGS: its workgroups per (batch, head), 0 = chosen here
     int fwd_cu_flip;     // MXD_MSDA_FWD_CU_FLIP: 1 = half of its wavefronts gather from LDS first, the others from memory
-                         // first; 0 = all in the same order (sums then formed in the general kernel's order, bit for bit)
+                         // first; 0 = all in the same order (sums then formed in the general kernel's order, bit for bit);
+                         // -1 = chosen here
     int bwd_fill_kernel; // MXD_MSDA_BWD_FILL_KERNEL: 1 = zero-fill by a kernel of its own
     int tile_order;      // MXD_MSDA_TILE_ORDER: 1 = work items of the tile pass batch-major, 0 = item-major, -1 = chosen here
     int bwd_sparse;      // MXD_MSDA_BWD_SPARSE: 0 = zero-fill (and, for 16-bit dtypes, round) the whole fp32 image of
@@ -104,7 +105,7 @@ void read_tuning()
     t.fwd_ahead = env_int("MXD_MSDA_FWD_AHEAD", 1);
     t.fwd_cu = env_int("MXD_MSDA_FWD_CU", -1);
     t.fwd_cu_wgs = env_int("MXD_MSDA_FWD_CU_WGS", 0);
-    t.fwd_cu_flip = env_int("MXD_MSDA_FWD_CU_FLIP", 1);
+    t.fwd_cu_flip = env_int("MXD_MSDA_FWD_CU_FLIP", -1);
     t.bwd_fill_kernel = env_int("MXD_MSDA_BWD_FILL_KERNEL", 0);
     t.tile_order = env_int("MXD_MSDA_TILE_ORDER", -1);
     t.bwd_lane_bytes = env_int("MXD_MSDA_BWD_LANE_BYTES", 0);
@@ -543,6 +544,16 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
     return true;
 }
 
+// Whether half of the wavefronts of the forward's one-workgroup-per-CU form work through their chunks from the LDS
+// groups on, so that memory gathers and LDS gathers of a CU's wavefronts run side by side.  Measured at the encoder
+// shape (alternating launches, one box): float16 70.9 -> 69.0 us -- 16 rows of 64 bytes per load instruction keep the
+// vector-memory pipeline twice as long as 8 rows of 128 bytes --, float32 78.9 -> 79.8 us: by default for 16-bit rows.
+int forward_cu_flip(int dtype)
+{
+    const int v = tuning().fwd_cu_flip;
+    return v >= 0 ? (v != 0) : (elem_size(dtype) == 2);
+}
+
 // level_cache: in/out, bytes of LDS for the forward's level cache (asked for -> granted)
 // cu_form: in/out, whether the forward may take / takes the one-workgroup-per-CU form
 int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_plan* p, int* level_cache = nullptr,
@@ -759,7 +770,7 @@ static int forward_common(int kind, const void* value, const int32_t* spatial_sh
     a.grid_w = (int32_t)grid_w;
     a.lds_cache_bytes = cache;
     a.fwd_ahead = tuning().fwd_ahead;
-    a.fwd_cu_flip = tuning().fwd_cu_flip;
+    a.fwd_cu_flip = forward_cu_flip(dtype);
     const hipError_t e = cu ? mxd::launch_forward_cu(dtype, a, static_cast<hipStream_t>(hip_stream))
                             : mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(e));
@@ -846,7 +857,7 @@ int mxd_msda_fused_forward(const void* value, const int32_t* spatial_shapes, con
     a.ref_dim = ref_dim;
     a.out = output;
     a.lds_cache_bytes = cache;
-    a.fwd_cu_flip = tuning().fwd_cu_flip;
+    a.fwd_cu_flip = forward_cu_flip(dtype);
     const hipError_t e = cu ? mxd::launch_forward_cu(dtype, a, static_cast<hipStream_t>(hip_stream))
                             : mxd::launch_forward(dtype, a, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(MXD_E_LAUNCH, "mxd_msda_fused_forward: launch failed: %s", hipGetErrorString(e));

@@ -739,9 +739,10 @@ def test_random_small_problems_16bit(gpu_device, seed):
                                         ("head_dim_128", torch.bfloat16)])
 def test_forward_cu_form_equals_the_general_form_at_full_size(gpu_device, monkeypatch, name, dtype):
     """The forward's one-workgroup-per-CU form (last levels in LDS, sample values handed across lanes by DPP; rows of 8,
-    4 and 16 lanes here) at the benchmark shapes: the encoder shape takes it by default, the others are made to.  Its
-    sums run in the same order as the general kernel's, so at full size the two must agree bit for bit; the general
-    kernel is checked against the oracle at these sizes elsewhere."""
+    4 and 16 lanes here) at the benchmark shapes: the encoder shape takes it by default, the others are made to.  With
+    every wavefront working through its chunks in the same order (MXD_MSDA_FWD_CU_FLIP=0) its sums run in the order of
+    the general kernel's, so at full size the two must agree bit for bit; the general kernel is checked against the
+    oracle at these sizes elsewhere."""
     from drivingsdk_amd import _C
     d = to_device(workloads.make_inputs(name, dtype=dtype), gpu_device)
     args = (d.value, d.spatial_shapes, d.level_start_index, d.sampling_locations, d.attention_weights)
@@ -750,13 +751,22 @@ def test_forward_cu_form_equals_the_general_form_at_full_size(gpu_device, monkey
     code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
     if name == "detr_encoder":
         assert _lib.make_plan(0, code, *dims).block == 1024, "the encoder shape is meant to take this form by default"
-    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=1)
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=1, MXD_MSDA_FWD_CU_FLIP=0)
     assert _lib.make_plan(0, code, *dims).block == 1024
     out_cu = _C.multi_scale_deformable_attn(*args)
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=1, MXD_MSDA_FWD_CU_FLIP=1)
+    out_flipped = _C.multi_scale_deformable_attn(*args)
     set_tuning(monkeypatch, MXD_MSDA_FWD_CU=0)
     assert _lib.make_plan(0, code, *dims).block != 1024
     out_general = _C.multi_scale_deformable_attn(*args)
     assert torch.equal(out_cu, out_general)
+    # Half of the wavefronts of the default build work through a chunk from its LDS groups on (MXD_MSDA_FWD_CU_FLIP=1):
+    # their units' sums are formed in another order, so they agree to rounding, not bit for bit
+    if dtype == torch.float32:
+        check_close(out_flipped.double().cpu().numpy(), out_general.double().cpu().numpy(), FWD_FP32, "output, flipped order")
+    else:
+        check_16bit(out_flipped.double().cpu().numpy(), out_general.double().cpu().numpy(), dtype, "output, flipped order",
+                    tol32=FWD_FP32)
 
 
 @pytest.mark.parametrize("seed", range(24))
@@ -793,7 +803,11 @@ def test_random_small_problems_cu_form(gpu_device, monkeypatch, seed):
     with monkeypatch.context() as m:
         set_tuning(m, MXD_MSDA_FWD_CU=0)
         general = run_gpu(inp, gpu_device, with_grads=False)[0]
-    assert np.array_equal(np.asarray(got), np.asarray(general))
+    with monkeypatch.context() as m:
+        set_tuning(m, MXD_MSDA_FWD_CU=1, MXD_MSDA_FWD_CU_WGS=1 + seed % 5, MXD_MSDA_FWD_CU_FLIP=0)
+        unflipped = run_gpu(inp, gpu_device, with_grads=False)[0]
+    # (the same order of summation in every wavefront: bit for bit the general kernel's result)
+    assert np.array_equal(np.asarray(unflipped), np.asarray(general))
 
 
 def test_backward_with_more_tiles_than_the_lds_bookkeeping_holds(gpu_device):
