@@ -269,7 +269,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                 merge_pair_records_in_quad(have, key, za, zb, keep);
 #pragma unroll
                 for (int r = 0; r < 2; ++r)
-                    if (keep[r]) atomicAdd(&cursor[tile_first[l] + ((key[r] - lvl[l].z) >> kTilePxLog2)], 1);
+                    if (keep[r]) atomicAdd(&cursor[tile_first[l] + ((key[r] - lvl[l].z) >> a.tile_px_log2)], 1);
             }
         };
         if constexpr (kUnroll == kLaneSamples) {
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             int32_t first = 0;
             for (int l = 0; l < a.nl; ++l) {
                 int32_t px;
-                const int32_t nt = level_tile_count(lvl[l].x, lvl[l].y, lvl[l].z, a.nk, &px);
+                const int32_t nt = level_tile_count(lvl[l].x, lvl[l].y, lvl[l].z, a.nk, a.tile_px_log2, &px);
                 const bool fits = first + nt <= a.tbl_stride - 1;
                 tile_first[l] = fits ? first : -1;
                 if (fits) first += nt;
@@ -351,7 +351,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             merge_pair_records_in_quad(have, key, za, zb, keep);
 #pragma unroll
             for (int r = 0; r < 2; ++r)
-                if (keep[r]) atomicAdd(&cursor[tile_first[l] + ((key[r] - lvl[l].z) >> kTilePxLog2)], 1);
+                if (keep[r]) atomicAdd(&cursor[tile_first[l] + ((key[r] - lvl[l].z) >> a.tile_px_log2)], 1);
         }
         __syncthreads();
         if (wave == 0) {
@@ -408,6 +408,16 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         const int total = cursor[a.tbl_stride - 1];  // (exclusive prefix: the entry after the last tile holds the sum)
         for (int i = threadIdx.x; i < total; i += blockDim.x) store_record(i, *rec_lds(i));
     };
+    // A workgroup that makes several passes (iterations, or chunks of units with more than 16 samples) and whose slab
+    // is small collects its records, 12 bytes each, in a buffer of its own behind the counters and writes the slab in
+    // whole lines when it is done: a pass adds a few records to every run, and stored one by one those pieces -- the
+    // shorter, the smaller the tiles of the grad_value pass are -- reach memory as partial lines.
+    typedef uint32_t __attribute__((may_alias)) u32_alias;
+    u32_alias* recbuf = nullptr;
+    if constexpr (!SCATTER) {
+        if (!rec_in_lds && a.rec_lds_bytes != 0)
+            recbuf = reinterpret_cast<u32_alias*>(smem + ((reinterpret_cast<unsigned char*>(cursor + a.tbl_stride) - smem + 15) & ~(size_t)15));
+    }
 
     for (int it = 0; it < a.plan.iters; ++it) {
         const int q0 = wk.q_begin + (((it * a.plan.waves_per_block + wave) * U) >> sp);
@@ -655,12 +665,19 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     for (int r = 0; r < 2; ++r) {
                         if (rec_keep[r]) {
                             const int32_t pos =
-                                atomicAdd(&cursor[tile_first[rec_l] + ((rec_key[r] - lvl[rec_l].z) >> kTilePxLog2)], 1);
-                            const uint32_t in_tile = (uint32_t)(rec_key[r] - lvl[rec_l].z) & (uint32_t)(kTilePx - 1);
-                            const u32x4 rec = {in_tile | ((uint32_t)(q - wk.q_begin) << kTilePxLog2),
+                                atomicAdd(&cursor[tile_first[rec_l] + ((rec_key[r] - lvl[rec_l].z) >> a.tile_px_log2)], 1);
+                            const uint32_t in_tile = (uint32_t)(rec_key[r] - lvl[rec_l].z) & ((1u << a.tile_px_log2) - 1u);
+                            const u32x4 rec = {in_tile | ((uint32_t)(q - wk.q_begin) << a.tile_px_log2),
                                                __builtin_bit_cast(uint32_t, rec_wa[r]), __builtin_bit_cast(uint32_t, rec_wb[r]), 0u};
-                            if (rec_in_lds) *rec_lds(pos) = rec;
-                            else store_record(pos, rec);
+                            if (rec_in_lds) {
+                                *rec_lds(pos) = rec;
+                            } else if (recbuf != nullptr) {
+                                recbuf[3 * pos] = rec.x;
+                                recbuf[3 * pos + 1] = rec.y;
+                                recbuf[3 * pos + 2] = rec.z;
+                            } else {
+                                store_record(pos, rec);
+                            }
                         }
                     }
                 }
@@ -684,6 +701,18 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     gloc[2 * e + 1] = from_f32<T>(0.f);
                 }
             }
+        }
+    }
+    if constexpr (!SCATTER) {
+        if (recbuf != nullptr) {  // (uniform over the workgroup; every wavefront leaves the loop above)
+            __syncthreads();
+            // the slab as it lies in the buffer: 16 bytes per lane, then the odd words
+            const int words = 3 * cursor[a.tbl_stride - 1], quads = words >> 2;
+            for (int i = threadIdx.x; i < quads; i += blockDim.x)
+                __builtin_amdgcn_raw_buffer_store_b128(u32x4{recbuf[4 * i], recbuf[4 * i + 1], recbuf[4 * i + 2], recbuf[4 * i + 3]}, sres,
+                                                       (uint32_t)i * 16u, 0, 2);
+            for (int i = 4 * quads + threadIdx.x; i < words; i += blockDim.x)
+                __builtin_amdgcn_raw_buffer_store_b32(recbuf[i], sres, (uint32_t)i * 4u, 0, 2);
         }
     }
 }

@@ -10,9 +10,13 @@
 // makes a per-sample scatter cost milliseconds.  Integer LDS atomics, plain LDS traffic and
 // registers are fast, so the scatter is turned inside out:
 //
-//   * The pixels of every level are cut into tiles of kTilePx pixels.  A workgroup owns one
-//     tile of one (batch, head); every group of 8 lanes owns 8 pixels of the tile and keeps
-//     their channels in registers for the whole kernel.
+//   * The pixels of every level are cut into tiles.  A workgroup (512 threads) owns one tile of
+//     one (batch, head); every thread keeps 32 sums in registers for the whole kernel: a group
+//     of 8 lanes owns 8 consecutive pixels of up to 32 channels (tiles of 512 pixels), 4 pixels
+//     of up to 64 channels (256) or 2 pixels of up to 128 channels (128), lane j holding
+//     channels 4j..4j+3 of every 32-channel block of each -- so that the records are streamed
+//     and the lists built and walked once whatever head_dim is (heads of more than 128
+//     channels take two passes over 128-pixel tiles).
 //   * The backward's first kernel leaves its samples as pair records {pixel, query, weight,
 //     weight of the pixel to the right}, sorted by tile inside the slab of each of its
 //     workgroups, with a table of run starts.  The owner of a tile streams the runs of its
@@ -39,7 +43,6 @@
 
 namespace mxd {
 
-constexpr int kWalk = 2; // lists a lane group walks together, one entry of each per trip
 
 // Work item table, evaluated identically by every workgroup.
 struct TileItem {
@@ -64,7 +67,7 @@ struct LevelInfo {
     {
         const i32x4 L = load_level(a, l);
         int32_t P, w = 0;
-        const int32_t n = level_tile_count(L.x, L.y, L.z, a.nk, &P);
+        const int32_t n = level_tile_count(L.x, L.y, L.z, a.nk, a.tile_px_log2, &P);
         H[l] = L.x;
         W[l] = L.y;
         base[l] = L.z;
@@ -83,7 +86,7 @@ struct LevelInfo {
             const int64_t p = (int64_t)H[l] * W[l];
             next += p;
             if (next > a.nk) return false;
-            tiles += (int32_t)((p + kTilePx - 1) >> kTilePxLog2);
+            tiles += (int32_t)((p + ((int64_t)1 << a.tile_px_log2) - 1) >> a.tile_px_log2);
         }
         return next == a.nk && tiles <= a.tbl_stride - 1;
     }
@@ -120,8 +123,9 @@ __device__ inline bool decode_tile_item(const KArgs& a, const TileArgs& t, const
             out->H = lv.H[l];
             out->W = lv.W[l];
             out->base = base;
-            out->p0 = base + ti * kTilePx;
-            out->p1 = (out->p0 + kTilePx) < (base + P) ? (out->p0 + kTilePx) : (base + P);
+            const int32_t tile_px = 1 << a.tile_px_log2;
+            out->p0 = base + ti * tile_px;
+            out->p1 = (out->p0 + tile_px) < (base + P) ? (out->p0 + tile_px) : (base + P);
             out->w0 = ci * wpc;
             out->w1 = (out->w0 + wpc) < a.nwg ? (out->w0 + wpc) : a.nwg;
             out->tile = lv_first[l] + ti;
@@ -147,7 +151,7 @@ __device__ inline void add_levels_without_tiles(const KArgs& a, int b, int h, in
         for (int l = 0; l < a.nl; ++l) {
             const i32x4 L = load_level(a, l);
             int32_t P;
-            const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, &P);
+            const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, a.tile_px_log2, &P);
             const bool fits = first + nt <= a.tbl_stride - 1;
             unfit[l] = fits ? 0 : 1;
             if (fits) first += nt;
@@ -180,18 +184,28 @@ __device__ inline void add_levels_without_tiles(const KArgs& a, int b, int h, in
     }
 }
 
-// CH = channels a lane group accumulates per pass (registers); heads with more channels are
-// done in several passes over the same records.  VEC = elements per load of a grad_out row.
-template <typename T, int CH, int VEC>
-__global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArgs a, const TileArgs t)
+// CHL = channels a lane accumulates per pass, 4 per 32-channel block of the row: 4, 8 or 16, for tiles of 512, 256 or
+// 128 pixels (32 sums per lane either way); heads with more than 8 * CHL channels are done in several passes over the
+// same records.  VEC = elements per load of a grad_out row.
+template <typename T, int CHL, int VEC>
+__global__ __launch_bounds__(kTileThreads, 4) void msda_gradv_tiles_kernel(const KArgs a, const TileArgs t)
 {
-    constexpr int CHL = CH / kLpp;                      // channels per lane
-    static_assert(CHL == 4 && 4 % VEC == 0, "a lane owns one 4-channel piece of a row");
-    constexpr int NW = kTilePx / kWave;                 // wavefronts per workgroup
+    static_assert((CHL == 4 || CHL == 8 || CHL == 16) && 4 % VEC == 0, "a lane owns one 4-channel piece of every 32-channel block");
+    constexpr int CH = kLpp * CHL;                      // channels per pass
+    constexpr int NB = CHL / 4;                         // 32-channel blocks per pass
+    constexpr int PPG = 32 / CHL;                       // pixels per lane group
+    constexpr int kTilePx = (kTileThreads / kLpp) * PPG;  // pixels per tile = pixel slots of the workgroup
+    constexpr int kTilePxLog2 = CHL == 4 ? 9 : CHL == 8 ? 8 : 7;
+    static_assert((1 << kTilePxLog2) == kTilePx, "tile size");
+    // lists a lane group walks together, one entry of each per trip (two trips are in flight: with 16 channels per
+    // lane one list's rows take the registers that two lists' take otherwise)
+    constexpr int kWalk = CHL >= 16 ? 1 : 2;
+    constexpr int NW = kTileThreads / kWave;            // wavefronts per workgroup
     constexpr uint32_t kDummyOfWave = kTileEntCap - 1;  // last entry slot of every wavefront
-    constexpr int kSlotPxAt = 32 * CH / 4;              // first entry behind wavefront 0's transposition scratch
-    static_assert(kSlotPxAt + kTilePx * 2 / 16 <= (int)kDummyOfWave, "slot map must fit wavefront 0's entry storage");
-    __shared__ uint32_t heads[kTilePx];                 // list head per pixel (entry index)
+    // (a wavefront transposes the sums of half of its lane groups at a time: 4 groups x 32 sums x 8 lanes = 4 KiB)
+    constexpr int kSlotPxAt = 4 * PPG * CH / 4;         // first entry behind wavefront 0's transposition scratch
+    static_assert(kSlotPxAt + kTileThreads * 2 / 16 <= (int)kDummyOfWave, "slot map must fit wavefront 0's entry storage");
+    __shared__ uint32_t heads[kTileThreads];            // list head per pixel slot (entry index)
     // entry: {byte offset of the grad_out row, weight for the list's pixel, weight for the
     // next pixel, next entry of the same list}
     __shared__ u32x4 ent[NW * kTileEntCap];
@@ -206,9 +220,10 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     // lists in the slots of the workgroup that no pixel of the tile uses -- when there are such slots.  The first
     // round counts entries per slot (two 16-bit counters per word); after it the same array holds, per slot,
     // {first extra slot, number of extra slots (2^k - 1)} as 9 + 4 bits.
-    __shared__ uint32_t slot_info[kTilePx / 2];
+    __shared__ uint32_t slot_info[kTileThreads / 2];
     __shared__ uint32_t spare_next, round1_total;
 
+    if (a.tile_px_log2 != kTilePxLog2) return;  // (uniform; the launcher derives both from head_dim)
     Work wk;
     if (!decode_block(t.map, blockIdx.x, a.bs, a.nh, t.items_per_bh, &wk)) return;
     if (t.batch_major == 0) {
@@ -227,9 +242,10 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     static_assert(sizeof(LevelInfo) <= sizeof(u32x4) * kTileEntCap, "the level values must fit one wavefront's entry storage");
     LevelInfo& lv_info = *reinterpret_cast<LevelInfo*>(&ent[0]);
     if ((int)threadIdx.x < a.nl) lv_info.fill(a, (int)threadIdx.x);
-    if (threadIdx.x < kTilePx / 2) slot_info[threadIdx.x] = 0;
-    // an empty list points at the dummy entry of the wavefront that owns the pixel
-    heads[threadIdx.x] = (threadIdx.x >> 6) * kTileEntCap + kDummyOfWave;
+    if (threadIdx.x < kTileThreads / 2) slot_info[threadIdx.x] = 0;
+    // an empty list points at the dummy entry of the wavefront that owns the pixel slot (slot s belongs to lane group
+    // s / PPG, i.e. to wavefront s / (8 PPG); slots past the tile size are never used)
+    heads[threadIdx.x] = (threadIdx.x / (kLpp * PPG)) % NW * kTileEntCap + kDummyOfWave;
     __syncthreads();
     if (threadIdx.x == 0) {
         item_ok = decode_tile_item(a, t, lv_info, wk.q_begin, &item_s, lv_first, lv_nt) ? 1 : 0;
@@ -248,14 +264,14 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     const int npx = it.p1 - it.p0;
     // A tile much smaller than the workgroup is held in several copies (lists and registers),
     // each taking the samples of some queries; the copies meet in the image through atomics.
-    const int npx_pad = (npx + kLpp - 1) / kLpp * kLpp;
+    const int npx_pad = (npx + PPG - 1) / PPG * PPG;
     int copies = 1;
     while (copies < 8 && 2 * copies * npx_pad <= kTilePx) copies *= 2;
     const bool owned = it.exclusive && copies == 1;  // plain stores are enough
     const int copies_log2 = __builtin_ctz(copies);
     const int nused = copies * npx_pad;              // slots that stand for a pixel of the tile
     const int nspare = kTilePx - nused;              // slots free for extra lists
-    const bool can_split = nspare >= kLpp;
+    const bool can_split = nspare >= PPG;
     // (owned && !can_split is what tile_stored_directly() says of this tile)
     const bool direct_t = a.sparse != 0 && a.grad_value_t != nullptr && owned && !can_split;
     typedef uint16_t __attribute__((may_alias)) u16_alias;  // halves of LDS words that are also accessed whole
@@ -288,18 +304,21 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
     const uint32_t dummy = seg + kDummyOfWave;
     if (lane == 0) ent[dummy] = u32x4{kInvalidCorner, 0u, 0u, dummy};
 
-    // lane j of group g = tid/kLpp keeps channels 4j..4j+3 of the pixels g*kLpp .. g*kLpp+kLpp-1
+    // lane j of group g = tid / 8 keeps channels 32k + 4j .. 32k + 4j + 3 (k < NB) of the pixels g*PPG .. g*PPG + PPG - 1
     const int grp = tid / kLpp, j = tid % kLpp;
 
     for (int cb = 0; cb < hd; cb += CH) {
-        float acc[kLpp][CHL];
+        float acc[PPG][CHL];
 #pragma unroll
-        for (int i = 0; i < kLpp; ++i)
+        for (int i = 0; i < PPG; ++i)
 #pragma unroll
             for (int c = 0; c < CHL; ++c) acc[i][c] = 0.0f;
         // channels past head_dim re-read channel 0; their sums are never written out
-        const int my_ch = cb + j * 4;
-        const uint32_t lane_off = ghead_off + (uint32_t)(my_ch < hd ? my_ch : 0) * (uint32_t)sizeof(T);
+        const int my_ch = cb + j * 4;  // (first channel of this lane in block 0; block k: + 32 k)
+        uint32_t lane_off[NB];
+#pragma unroll
+        for (int k = 0; k < NB; ++k)
+            lane_off[k] = ghead_off + (uint32_t)(my_ch + 32 * k < hd ? my_ch + 32 * k : 0) * (uint32_t)sizeof(T);
         const int nch = (hd - cb) < CH ? (hd - cb) : CH;
 
         // input state of this wavefront (uniform): next group of runs, records of the current
@@ -380,7 +399,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     wb = __builtin_bit_cast(float, za);
                     const int copy_off = (int)(q & (uint32_t)(copies - 1)) * npx_pad;
                     const bool in_r = pl + 1 < npx;
-                    const bool pair = in_r && (pl % kLpp) != kLpp - 1;
+                    const bool pair = in_r && (pl % PPG) != PPG - 1;
                     lst[0] = pl + copy_off;
                     w0[0] = wa;
                     w1[0] = pair ? wb : 0.0f;
@@ -437,9 +456,9 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     smask &= smask - 1;
                     const uint32_t sq = __builtin_amdgcn_readlane(q, src_lane);
                     const float sw = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(uint32_t, wb), src_lane));
-                    if (lane < nch) {
-                        const float g = to_f32(gout[((int64_t)wk.b * a.nq + sq) * row_pitch + (int64_t)wk.h * hd + cb + lane]);
-                        unsafeAtomicAdd(gimg + (int64_t)it.p1 * row_pitch + (int64_t)wk.h * hd + cb + lane, sw * g);
+                    for (int ch = lane; ch < nch; ch += kWave) {
+                        const float g = to_f32(gout[((int64_t)wk.b * a.nq + sq) * row_pitch + (int64_t)wk.h * hd + cb + ch]);
+                        unsafeAtomicAdd(gimg + (int64_t)it.p1 * row_pitch + (int64_t)wk.h * hd + cb + ch, sw * g);
                     }
                 }
             }
@@ -469,9 +488,9 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 first_round = false;
             }
 
-            // ---- every group of kLpp lanes walks the lists of its kLpp pixels -----------------
-            // The lanes of a group read one grad_out row with ONE coalesced load (lane j: channels
-            // 4j..4j+3): the memory pipeline's cost is per cache line touched by an instruction.
+            // ---- every group of 8 lanes walks the lists of its PPG pixels ----------------------
+            // The lanes of a group read a 32-channel block of a grad_out row with ONE coalesced load (lane j:
+            // channels 4j..4j+3 of the block): the memory pipeline's cost is per cache line touched by an instruction.
             // The loop body is branch-free: a list that has ended keeps "reading" the dummy entry.
             // kWalk lists are walked together, one entry of each per trip, and two trips are in flight.
             {
@@ -482,17 +501,20 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                     wa = __builtin_bit_cast(float, ya);
                     wb = __builtin_bit_cast(float, za);
 #pragma unroll
-                    for (int c = 0; c < 4; c += VEC) {
-                        float g1[VEC];
-                        RowIO<T, VEC>::unpack(RowIO<T, VEC>::load_raw(gres, en.x + lane_off + (uint32_t)(c * sizeof(T))), g1);
+                    for (int k = 0; k < NB; ++k) {
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) g[c + v] = g1[v];
+                        for (int c = 0; c < 4; c += VEC) {
+                            float g1[VEC];
+                            RowIO<T, VEC>::unpack(RowIO<T, VEC>::load_raw(gres, en.x + lane_off[k] + (uint32_t)(c * sizeof(T))), g1);
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) g[4 * k + c + v] = g1[v];
+                        }
                     }
                     e = en.w;
                 };
 #pragma unroll
-                for (int i = 0; i < kLpp; i += kWalk) {
-                    const int px = grp * kLpp + i;
+                for (int i = 0; i < PPG; i += kWalk) {
+                    const int px = grp * PPG + i;
                     uint32_t e[kWalk];
 #pragma unroll
                     for (int m = 0; m < kWalk; ++m) e[m] = heads[px + m];
@@ -510,8 +532,8 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
 #pragma unroll
                             for (int c = 0; c < CHL; ++c) {
                                 acc[i + m][c] = __builtin_fmaf(u[m], g[m][c], acc[i + m][c]);
-                                if (i + m + 1 < kLpp)
-                                    acc[(i + m + 1) % kLpp][c] = __builtin_fmaf(v[m], g[m][c], acc[(i + m + 1) % kLpp][c]);
+                                if (i + m + 1 < PPG)
+                                    acc[(i + m + 1) % PPG][c] = __builtin_fmaf(v[m], g[m][c], acc[(i + m + 1) % PPG][c]);
                             }
                         }
                     };
@@ -565,14 +587,17 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
         }
         if (owned && !split && t.store_vec == 4) {
             // the lanes of a group hold a whole row of each of their pixels: 16-byte stores
-            if (my_ch < hd) {
 #pragma unroll
-                for (int i = 0; i < kLpp; ++i) {
-                    const int px = grp_w * kLpp + i;
+            for (int kb = 0; kb < NB; ++kb) {
+                const int ch_w = my_ch + 32 * kb;
+                if (ch_w >= hd) continue;
+#pragma unroll
+                for (int i = 0; i < PPG; ++i) {
+                    const int px = grp_w * PPG + i;
                     if (px < npx) {
                         f32x4* dst = reinterpret_cast<f32x4*>(gimg + (int64_t)(it.p0 + px) * row_pitch +
-                                                              (int64_t)wk.h * hd + my_ch);
-                        f32x4 v = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+                                                              (int64_t)wk.h * hd + ch_w);
+                        f32x4 v = {acc[i][4 * kb + 0], acc[i][4 * kb + 1], acc[i][4 * kb + 2], acc[i][4 * kb + 3]};
                         if (px == 0) {
                             // the first pixel of a tile also receives, through atomics, the right
                             // halves of pairs that start on the last pixel of the previous tile
@@ -587,7 +612,7 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                             __builtin_nontemporal_store(r, reinterpret_cast<t4*>(static_cast<T*>(a.grad_value_t) +
                                                                                  (size_t)wk.b * (a.gbatch_bytes / 4) +
                                                                                  (int64_t)(it.p0 + px) * row_pitch +
-                                                                                 (int64_t)wk.h * hd + my_ch));
+                                                                                 (int64_t)wk.h * hd + ch_w));
                         } else {
                             if (t.accumulate) v += *dst;
                             // (non-temporal: nothing reads these rows again before the kernel ends; backward 283.8 ->
@@ -601,9 +626,9 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
             // Rows shared with other workgroups (tiles split by query range) are added with
             // atomics, which the memory side carries out per 64-byte request: pass the registers
             // through LDS (the entry storage, free after the last round) so that consecutive
-            // lanes hold consecutive floats of a row.  32 pixels at a time.
+            // lanes hold consecutive floats of a row.  Four lane groups (4 PPG pixel slots, 1024 sums) at a time.
             typedef uint32_t __attribute__((may_alias)) u32_alias;
-            static_assert(32 * CH * 4 <= kTileEntCap * 16, "transposition scratch must fit the entry storage");
+            static_assert(4 * PPG * CH * 4 <= kTileEntCap * 16, "transposition scratch must fit the entry storage");
             u32x4* tr4 = &ent[seg];
             const u32_alias* tr1 = reinterpret_cast<const u32_alias*>(tr4);
             for (int half = 0; half < 2; ++half) {
@@ -611,15 +636,17 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
                 if (((lane_w / kLpp) >> 2) == half) {
                     const int gl = (lane_w / kLpp) & 3;
 #pragma unroll
-                    for (int i = 0; i < kLpp; ++i)
-                        tr4[(gl * kLpp + i) * (CH / 4) + j] =
-                            u32x4{__builtin_bit_cast(uint32_t, acc[i][0]), __builtin_bit_cast(uint32_t, acc[i][1]),
-                                  __builtin_bit_cast(uint32_t, acc[i][2]), __builtin_bit_cast(uint32_t, acc[i][3])};
+                    for (int i = 0; i < PPG; ++i)
+#pragma unroll
+                        for (int kb = 0; kb < NB; ++kb)
+                            tr4[(gl * PPG + i) * (CH / 4) + 8 * kb + j] =
+                                u32x4{__builtin_bit_cast(uint32_t, acc[i][4 * kb + 0]), __builtin_bit_cast(uint32_t, acc[i][4 * kb + 1]),
+                                      __builtin_bit_cast(uint32_t, acc[i][4 * kb + 2]), __builtin_bit_cast(uint32_t, acc[i][4 * kb + 3])};
                 }
                 wave_lds_sync();
-                const int px_base = wave * kWave + half * 32;
+                const int px_base = wave * (kLpp * PPG) + half * (4 * PPG);
 #pragma unroll 4
-                for (int k = 0; k < 32 * CH / kWave; ++k) {
+                for (int k = 0; k < 4 * PPG * CH / kWave; ++k) {
                     const int idx = k * kWave + lane_w;
                     const int pl = idx / CH, c = idx % CH;
                     const int vp = px_base + pl;             // pixel slot of the workgroup
@@ -653,14 +680,22 @@ __global__ __launch_bounds__(kTilePx, 4) void msda_gradv_tiles_kernel(const KArg
 template <typename T>
 static hipError_t launch_t(const KArgs& a, const TileArgs& t, hipStream_t stream)
 {
-    // an octet of lanes reads a 32-channel slice of a grad_out row, 4 channels per lane: one
-    // load per lane when head_dim and the pointer alignment allow it
-    if (t.vec >= 4)
-        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 32, 4>), dim3(t.grid), dim3(t.block), 0, stream, a, t);
+    // an octet of lanes reads a 32-channel block of a grad_out row, 4 channels per lane: one
+    // load per lane when head_dim and the pointer alignment allow it; the wider forms (tiles of 256 and 128
+    // pixels) are built for that case only
+    const dim3 grid(t.grid), block(t.block);
+    if (a.tile_px_log2 == 8 && t.vec >= 4)
+        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 8, 4>), grid, block, 0, stream, a, t);
+    else if (a.tile_px_log2 == 7 && t.vec >= 4)
+        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 16, 4>), grid, block, 0, stream, a, t);
+    else if (a.tile_px_log2 != kTilePxLog2Max)
+        return hipErrorInvalidConfiguration;
+    else if (t.vec >= 4)
+        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 4, 4>), grid, block, 0, stream, a, t);
     else if (t.vec == 2)
-        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 32, 2>), dim3(t.grid), dim3(t.block), 0, stream, a, t);
+        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 4, 2>), grid, block, 0, stream, a, t);
     else
-        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 32, 1>), dim3(t.grid), dim3(t.block), 0, stream, a, t);
+        hipLaunchKernelGGL((msda_gradv_tiles_kernel<T, 4, 1>), grid, block, 0, stream, a, t);
     return hipGetLastError();
 }
 

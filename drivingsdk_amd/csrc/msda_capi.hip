@@ -88,6 +88,9 @@ struct Tuning {
     int bwd_unit_split;  // MXD_MSDA_BWD_UNIT_SPLIT: 0 = a unit of the first backward kernel is always a whole query
     int bwd_lane_bytes;  // MXD_MSDA_BWD_LANE_BYTES: most bytes of a row one lane of the first backward kernel loads
                          // (16, 8, 4), 0 = chosen here
+    int tile_px_log2;    // MXD_MSDA_TILE_PX_LOG2: log2 of the pixels per tile of the grad_value pass (9, 8, 7), 0 = chosen here
+    int bwd_rec_lds;     // MXD_MSDA_BWD_REC_LDS: 0 = workgroups of the first backward kernel that make several passes store
+                         // their records one by one, 1 = they collect their slab in LDS wherever it fits, -1 = chosen here
 };
 Tuning g_tuning;
 std::once_flag g_tuning_once;
@@ -111,6 +114,8 @@ void read_tuning()
     t.bwd_lane_bytes = env_int("MXD_MSDA_BWD_LANE_BYTES", 0);
     t.bwd_sparse = env_int("MXD_MSDA_BWD_SPARSE", 1);
     t.bwd_unit_split = env_int("MXD_MSDA_BWD_UNIT_SPLIT", 1);
+    t.tile_px_log2 = env_int("MXD_MSDA_TILE_PX_LOG2", 0);
+    t.bwd_rec_lds = env_int("MXD_MSDA_BWD_REC_LDS", -1);
     g_tuning = t;
 }
 
@@ -290,6 +295,7 @@ static int64_t bwd_tile_q(int dtype, const Dims& d)
 }
 struct BwdLayout {
     bool tiles;          // false: one kernel with global atomics
+    int tile_px_log2;    // log2 of the pixels per tile of the grad_value pass
     int64_t tile_q;      // queries per workgroup of the first kernel
     int64_t nwg;         // workgroups of the first kernel per (batch, head)
     int64_t rec_cap;     // pair records per workgroup slab: 2 per sample
@@ -297,16 +303,38 @@ struct BwdLayout {
     size_t tbl_bytes, rec_bytes, image_bytes, total;
 };
 
-BwdLayout bwd_layout(int dtype, const Dims& d)
+// Pixels per tile of the grad_value pass, as a power of two: every thread of its workgroups keeps 32 sums, so 512 pixels
+// of up to 32 channels, 256 of up to 64, 128 of more (msda_plan.h).  The smaller tiles are built for rows that are read
+// four elements per lane (`wide_rows`: head_dim a multiple of 4 and pointers aligned for it); other rows keep 512-pixel
+// tiles and take one pass over the records per 32 channels.
+int preferred_tile_px_log2(const Dims& d, bool wide_rows)
+{
+    if (!wide_rows || d.hd % 4 != 0) return mxd::kTilePxLog2Max;
+    const int v = tuning().tile_px_log2;
+    if (v >= 7 && v <= mxd::kTilePxLog2Max) return v;
+    if (d.hd <= 32) return mxd::kTilePxLog2Max;
+    // Maps so small that a level is a tile of 512 pixels or less keep that tile and take two or four passes: the slots
+    // of the workgroup that the tile leaves free are what a pixel that collects far more entries than the others gets
+    // its extra lists from, and a tile cut in two has none (geometric kernel attention at 15 x 25 pixels and 64 channels,
+    // where clamping piles half of the samples on the border: 0.80 ms per step with one tile of 375 pixels and two
+    // passes, 0.90 ms with tiles of 256 + 119 pixels and one).
+    if (d.nk <= (int64_t)d.nl << mxd::kTilePxLog2Max) return mxd::kTilePxLog2Max;
+    // (measured at 8 heads x 128 channels, encoder levels: float16 backward 588 us with tiles of 512 pixels, 431 with 256,
+    //  383 with 128; float32 722, 590, 586)
+    return d.hd <= 64 ? 8 : 7;
+}
+
+BwdLayout bwd_layout_for(int dtype, const Dims& d, int tile_px_log2)
 {
     BwdLayout L;
     memset(&L, 0, sizeof(L));
+    L.tile_px_log2 = tile_px_log2;
     L.tile_q = bwd_tile_q(dtype, d);
     L.nwg = (d.nq + L.tile_q - 1) / L.tile_q;
     L.rec_cap = 2 * L.tile_q * d.nl * d.np;
-    // tiles per (batch, head) when the levels do not overlap: sum of ceil(pixels/kTilePx) <= nk/kTilePx + nl
+    // tiles per (batch, head) when the levels do not overlap: sum of ceil(pixels / tile) <= nk / tile + nl
     // (the kernels leave out levels that would not fit, which can only happen for overlapping levels)
-    L.tbl_stride = d.nk / mxd::kTilePx + d.nl + 1;
+    L.tbl_stride = (d.nk >> tile_px_log2) + d.nl + 1;
     const int64_t tbl = d.bs * d.nh * L.nwg * L.tbl_stride * 4;
     // dynamic LDS of the first kernel with the most units per wavefront the row can have (16-byte aligned pointers)
     int vec, lpr, npass;
@@ -325,6 +353,43 @@ BwdLayout bwd_layout(int dtype, const Dims& d)
     if (elem_size(dtype) == 2) L.image_bytes = (size_t)d.bs * d.nk * d.nh * d.hd * 4;
     L.total = L.tbl_bytes + L.rec_bytes + L.image_bytes;
     return L;
+}
+
+// The layout a launch uses: the tile size preferred for the rows, or 512-pixel tiles where the finer run table would
+// not fit the first kernel's bookkeeping.
+BwdLayout bwd_layout(int dtype, const Dims& d, bool wide_rows)
+{
+    const int pref = preferred_tile_px_log2(d, wide_rows);
+    BwdLayout L = bwd_layout_for(dtype, d, pref);
+    if (!L.tiles && pref != mxd::kTilePxLog2Max) L = bwd_layout_for(dtype, d, mxd::kTilePxLog2Max);
+    return L;
+}
+
+// Workspace a caller must bring: what the launch may need whichever way its pointers are aligned.
+size_t bwd_workspace_bytes(int dtype, const Dims& d)
+{
+    const size_t a = bwd_layout(dtype, d, true).total, b = bwd_layout(dtype, d, false).total;
+    return a > b ? a : b;
+}
+
+// LDS for the slab of a workgroup of the first backward kernel that makes several passes (msda_bwd.hip): 12 bytes per
+// record behind the counters, when the slab is small enough to leave four workgroups to a CU and the kernel stays
+// inside the default limit of dynamic LDS.  A workgroup that makes one pass of one chunk (the plain operator and the
+// fused form) collects its records in its staging strips instead.  Adds the bytes to the plan.
+int plan_record_buffer(mxd_msda_plan* p, const BwdLayout& L, const Dims& d, int dtype, bool plain_or_fused, int unit_split_log2)
+{
+    if (!L.tiles) return 0;
+    // By default for 16-bit rows only (MXD_MSDA_BWD_REC_LDS=1: wherever it fits).  Measured, backward at 8 heads x 128
+    // channels with tiles of 128 pixels: float16 414 -> 383 us; float32 586 -> 596 us, geometric kernel attention (64
+    // channels, float32) 0.80 -> 0.86 ms per step -- there the buffer costs the kernel a workgroup per CU, which weighs
+    // more than the partial lines.
+    if (tuning().bwd_rec_lds < 0 && elem_size(dtype) != 2) return 0;
+    const bool one_pass = plain_or_fused && p->iters == 1 && d.nl * d.np <= ((int64_t)mxd::kChunk << unit_split_log2);
+    const int64_t bytes = L.rec_cap * (mxd::kRecDwords * 4);
+    const int64_t total = (((int64_t)p->lds_bytes + 15) & ~(int64_t)15) + bytes;
+    if (one_pass || bytes > 24 * 1024 || total > 40 * 1024 || tuning().bwd_rec_lds == 0) return 0;
+    p->lds_bytes = (uint32_t)total;
+    return (int)bytes;
 }
 
 // Geometry of the tile-ownership grad_value kernel (msda_bwd_tiles.hip).
@@ -348,7 +413,7 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
         // step, 480 items 0.81 ms, 384 items 0.87 ms).  Pick the chunk count with the least estimated duration:
         // items in flight one after another x (records per item + about 8192 records' worth of start, statistics
         // round and write-out per item).
-        const int64_t nt = (d.nk + mxd::kTilePx - 1) / mxd::kTilePx;
+        const int64_t nt = (d.nk + (int64_t(1) << L.tile_px_log2) - 1) >> L.tile_px_log2;
         const int64_t per_tile = 2 * d.nq * d.np / nt;
         int64_t best_c = 1;
         double best_cost = -1.0;
@@ -378,7 +443,7 @@ int make_tile_args(const Dims& d, const BwdLayout& L, int vec, int accumulate, m
     const int64_t grid = fill_xcd_map(&t->map, d.bs, d.nh, t->items_per_bh);
     if (grid >= (int64_t(1) << 31)) return fail(MXD_E_SHAPE, "backward needs %lld workgroups, beyond the launch limit", (long long)grid);
     t->grid = (uint32_t)grid;
-    t->block = mxd::kTilePx;
+    t->block = mxd::kTileThreads;
     return MXD_OK;
 }
 
@@ -577,7 +642,7 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     p->waves_per_block = 4;
     int iters = tuning().fwd_iters;
     if (iters < 1) iters = 1;
-    const BwdLayout L = bwd_layout(dtype, d);
+    const BwdLayout L = bwd_layout(dtype, d, vec >= 4);
     // the tile pass wants L.tile_q queries per workgroup of the first backward kernel
     int split = 1;  // units of the backward's first kernel that share a query
     if (backward) {
@@ -870,7 +935,7 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
     take_meta_flag(&dtype);
     const Dims d{bs, nk, nh, hd, nl, nl_attn, nq, np};
     if (check_dims(dtype, d) != MXD_OK) return 0;
-    return bwd_layout(dtype, d).total;
+    return bwd_workspace_bytes(dtype, d);
 }
 
 // What the fused form adds to a backward call.
@@ -908,7 +973,13 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     if (fused && (!fused->ref || !fused->out)) return fail(MXD_E_NULL, "%s: NULL data pointer", who);
     if (fused && fused->ref_dim != 2 && fused->ref_dim != 4)
         return fail(MXD_E_SHAPE, "Last dim of reference_points must be 2 or 4, but get %d instead.", fused->ref_dim);
-    const BwdLayout L = bwd_layout(dtype, d);
+    int align = ptr_align(value);
+    if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
+    mxd::KArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = make_plan(1, dtype, d, align, &a.plan);
+    if (rc != MXD_OK) return rc;
+    const BwdLayout L = bwd_layout(dtype, d, a.plan.vec >= 4);  // (as make_plan laid the first kernel's LDS out)
     const size_t part_bytes = (fused && fused->grad_ref) ? fused_part_bytes(d, fused->ref_dim) : 0;
     const size_t need = L.total + part_bytes;
     if (need > 0 && (!workspace || workspace_bytes < need))
@@ -922,14 +993,10 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     char* ws = static_cast<char*>(workspace);
     float* image = half ? reinterpret_cast<float*>(ws + L.tbl_bytes + L.rec_bytes) : static_cast<float*>(grad_value);
     if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "%s: grad_value is not 4-byte aligned", who);
-    int align = ptr_align(value);
-    if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
-    mxd::KArgs a;
-    memset(&a, 0, sizeof(a));
-    rc = make_plan(1, dtype, d, align, &a.plan);
-    if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.tile_px_log2 = L.tile_px_log2;
     a.unit_split_log2 = unit_split_log2(a.plan);
+    a.rec_lds_bytes = plan_record_buffer(&a.plan, L, d, dtype, !gka && !grid, a.unit_split_log2);
     a.meta_i64 = meta64;
     a.value = value;
     a.shapes = spatial_shapes;
@@ -1003,7 +1070,7 @@ size_t mxd_msda_fused_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk
     take_meta_flag(&dtype);
     const Dims d{bs, nk, nh, hd, nl, nl, nq, np};
     if (check_dims(dtype, d) != MXD_OK || (ref_dim != 2 && ref_dim != 4)) return 0;
-    return bwd_layout(dtype, d).total + (want_grad_ref ? fused_part_bytes(d, ref_dim) : 0);
+    return bwd_workspace_bytes(dtype, d) + (want_grad_ref ? fused_part_bytes(d, ref_dim) : 0);
 }
 
 int mxd_msda_fused_backward(const void* value, const int32_t* spatial_shapes, const int32_t* level_start_index,
@@ -1131,7 +1198,7 @@ size_t mxd_dagg_backward_workspace_bytes(int dtype, int64_t bs, int64_t num_feat
     Dims d;
     if (dagg_dims(dtype, bs, num_feat, num_embeds, num_cams, num_scale, num_anchors, num_pts, num_groups, &d) != MXD_OK)
         return 0;
-    return bwd_layout(dtype, d).total + dagg_part_bytes(d, num_cams);
+    return bwd_workspace_bytes(dtype, d) + dagg_part_bytes(d, num_cams);
 }
 
 int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, const int32_t* scale_start_index,
@@ -1148,7 +1215,13 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     if (!mc_ms_feat || !spatial_shape || !scale_start_index || !sampling_location || !weights || !grad_output ||
         !grad_mc_ms_feat || !grad_sampling_location || !grad_weights)
         return fail(MXD_E_NULL, "mxd_dagg_backward: NULL data pointer");
-    const BwdLayout L = bwd_layout(dtype, d);
+    int align = ptr_align(mc_ms_feat);
+    if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
+    mxd::KArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = make_plan(1, dtype, d, align, &a.plan);
+    if (rc != MXD_OK) return rc;
+    const BwdLayout L = bwd_layout(dtype, d, a.plan.vec >= 4);  // (as make_plan laid the first kernel's LDS out)
     const size_t part_bytes = dagg_part_bytes(d, num_cams);
     const size_t need = L.total + part_bytes;
     if (!workspace || workspace_bytes < need)
@@ -1161,14 +1234,10 @@ int mxd_dagg_backward(const void* mc_ms_feat, const int32_t* spatial_shape, cons
     float* image = half ? reinterpret_cast<float*>(ws + L.tbl_bytes + L.rec_bytes) : static_cast<float*>(grad_mc_ms_feat);
     float* part = reinterpret_cast<float*>(ws + L.total);
     if (reinterpret_cast<uintptr_t>(image) & 3u) return fail(MXD_E_SHAPE, "mxd_dagg_backward: grad_mc_ms_feat is not 4-byte aligned");
-    int align = ptr_align(mc_ms_feat);
-    if (ptr_align(grad_output) < align) align = ptr_align(grad_output);
-    mxd::KArgs a;
-    memset(&a, 0, sizeof(a));
-    rc = make_plan(1, dtype, d, align, &a.plan);
-    if (rc != MXD_OK) return rc;
     fill_args(&a, dtype, d);
+    a.tile_px_log2 = L.tile_px_log2;
     a.unit_split_log2 = unit_split_log2(a.plan);
+    a.rec_lds_bytes = plan_record_buffer(&a.plan, L, d, dtype, false, a.unit_split_log2);
     a.meta_i64 = meta64;
     fill_dagg(&a, num_cams, num_scale);
     a.value = mc_ms_feat;

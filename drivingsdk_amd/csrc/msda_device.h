@@ -61,13 +61,16 @@ struct KArgs {
     // first kernel (tile_q queries of one (batch, head)) owns a slab of rec_cap pair records,
     // which it fills sorted by tile; row [w] of the table holds the start of every tile's run
     // inside slab w (tbl_stride entries, the last used one being the total).
-    // record (12 bytes) = {pixel within its tile | query within the workgroup << kTilePxLog2, weight of that pixel,
+    // record (12 bytes) = {pixel within its tile | query within the workgroup << tile_px_log2, weight of that pixel,
     //                      weight of the pixel to its right}
     uint32_t* rec;         // [bs*nh][nwg][rec_cap] records of kRecDwords dwords
     uint32_t* tbl;         // [bs*nh][nwg][tbl_stride]
     int32_t nwg;           // workgroups of the first kernel per (batch, head)
     int32_t rec_cap;       // 2 * tile_q * nl * np
     int32_t tbl_stride;    // upper bound of tiles per (batch, head), plus one
+    int32_t tile_px_log2;  // log2 of the pixels per tile of the grad_value pass (9, 8 or 7: see msda_plan.h)
+    int32_t rec_lds_bytes; // first backward kernel: LDS behind its counters (16-byte aligned) in which a workgroup that makes
+                           // several passes collects its slab before it writes it; 0 = none (records stored one by one)
     int32_t tile_target;   // pair records per work item of the tile pass aimed at when a hot tile is split by query range
     int32_t tile_max_chunks;  // most query chunks a tile is split into
     int32_t sparse;        // 1: only the rows of the image that receive atomic additions are zero-filled (and, for 16-bit
@@ -97,8 +100,11 @@ __device__ inline i32x4 load_level(const KArgs& a, int l)
 
 // ---- tiles of the grad_value pass, as every kernel of the backward sees them ---------------------------------------
 constexpr int kRecDwords = 3;  // dwords of a pair record
-constexpr int kLpp = 8;        // lanes per pixel row = pixels per lane group of the tile pass
+constexpr int kLpp = 8;        // lanes of a lane group of the tile pass (a group reads a row with one load per 32 channels)
 constexpr int kRowParts = 16;  // pieces a tile's rows are cut into for the zero-fill and the rounding
+
+// Pixels per lane group of the tile pass: 8 for tiles of 512 pixels, 4 for 256, 2 for 128 (64 groups per workgroup).
+__device__ inline int32_t tile_group_px(int32_t tile_px_log2) { return 1 << (tile_px_log2 - 6); }
 
 // Query chunks the tiles of a level with `nt` tiles are split into by the tile pass; *wpc: workgroups of the first
 // kernel per chunk.
@@ -127,9 +133,10 @@ __device__ inline int32_t level_tile_chunks(const KArgs& a, int32_t nt, int32_t*
 // them (the tile is not split by query range and is too full to be held in copies or to have slots left for extra
 // lists), except to the tile's first pixel, which also receives the right halves of pairs that start on the last
 // pixel of the tile before it.
-__device__ inline bool tile_stored_directly(int32_t chunks, int32_t npx)
+__device__ inline bool tile_stored_directly(int32_t chunks, int32_t npx, int32_t tile_px_log2)
 {
-    return chunks == 1 && kTilePx - ((npx + kLpp - 1) / kLpp * kLpp) < kLpp;
+    const int32_t g = tile_group_px(tile_px_log2);
+    return chunks == 1 && (1 << tile_px_log2) - ((npx + g - 1) / g * g) < g;
 }
 
 // Whether the levels tile the keys exactly and in order -- the first level starts at key 0, every other one where the
@@ -148,7 +155,7 @@ __device__ inline bool levels_tile_the_keys(const KArgs& a)
         const int64_t px = (int64_t)L.x * L.y;
         next += px;
         if (next > a.nk) return false;
-        tiles += (int32_t)((px + kTilePx - 1) >> kTilePxLog2);
+        tiles += (int32_t)((px + ((int64_t)1 << a.tile_px_log2) - 1) >> a.tile_px_log2);
     }
     return next == a.nk && tiles <= a.tbl_stride - 1;
 }
@@ -162,18 +169,18 @@ __device__ inline bool atomic_rows_of_part(const KArgs& a, int32_t tile, int32_t
     for (int l = 0; l < a.nl; ++l) {
         const i32x4 L = load_level(a, l);
         int32_t P;
-        const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, &P);
+        const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, a.tile_px_log2, &P);
         if (first + nt > a.tbl_stride - 1) continue;  // (a level that does not fit the run table has no tiles)
         if (tile < first + nt) {
-            const int32_t ti = tile - first;
-            const int32_t p0 = L.z + ti * kTilePx;
-            const int32_t npx = (P - ti * kTilePx) < kTilePx ? (P - ti * kTilePx) : kTilePx;
+            const int32_t ti = tile - first, tile_px = 1 << a.tile_px_log2;
+            const int32_t p0 = L.z + ti * tile_px;
+            const int32_t npx = (P - ti * tile_px) < tile_px ? (P - ti * tile_px) : tile_px;
             int32_t wpc;
-            if (tile_stored_directly(level_tile_chunks(a, nt, &wpc), npx)) {
+            if (tile_stored_directly(level_tile_chunks(a, nt, &wpc), npx, a.tile_px_log2)) {
                 *r0 = p0;
                 *r1 = part == 0 ? p0 + 1 : p0;
             } else {
-                constexpr int per = kTilePx / kRowParts;
+                const int per = tile_px / kRowParts;
                 *r0 = p0 + (part * per < npx ? part * per : npx);
                 *r1 = p0 + ((part + 1) * per < npx ? (part + 1) * per : npx);
             }

@@ -34,23 +34,27 @@ constexpr int kCuLdsBytes = 160 * 1024;
 constexpr int kCuWaves = 16;         // wavefronts of its workgroups
 constexpr int kCuTableBytes = 2 * (kMaxLevels + 1) * 16 + 32;  // its two level tables ahead of the cached rows (multiple of 64)
 
-constexpr int kTilePx = 512;         // pixels per tile of the grad_value pass = threads of its workgroups
-constexpr int kTilePxLog2 = 9;
+constexpr int kTileThreads = 512;    // threads of the workgroups of the grad_value pass
+// Pixels per tile of the grad_value pass: every thread of a workgroup keeps 32 sums, so a workgroup holds 512 pixels of
+// up to 32 channels, 256 of up to 64 or 128 of up to 128 (heads of more channels take two passes over 128-pixel tiles).
+// The launcher picks the size from head_dim (KArgs::tile_px_log2: 9, 8 or 7); the first backward kernel sorts its
+// records by tiles of that size.
+constexpr int kTilePxLog2Max = 9;
 
 struct Work {
     int32_t b, h, q_begin, q_end;
 };
 
 // Tiles of the grad_value pass that a level contributes: its pixels [base, base + H*W), clipped
-// to the value tensor, in pieces of kTilePx.  *pixels receives the clipped pixel count.
-MXD_HD inline int32_t level_tile_count(int32_t H, int32_t W, int32_t base, int32_t nk, int32_t* pixels)
+// to the value tensor, in pieces of 2^tile_px_log2.  *pixels receives the clipped pixel count.
+MXD_HD inline int32_t level_tile_count(int32_t H, int32_t W, int32_t base, int32_t nk, int32_t tile_px_log2, int32_t* pixels)
 {
     *pixels = 0;
     if (H <= 0 || W <= 0 || base < 0 || base >= nk) return 0;
     int64_t P = (int64_t)H * W;
     if (base + P > nk) P = nk - base;  // never address past the value tensor
     *pixels = (int32_t)P;
-    return (int32_t)((P + kTilePx - 1) >> kTilePxLog2);
+    return (int32_t)((P + ((int64_t)1 << tile_px_log2) - 1) >> tile_px_log2);
 }
 
 // Decode a workgroup index.  Returns false when the workgroup has nothing to do.

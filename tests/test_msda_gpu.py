@@ -678,6 +678,46 @@ def test_random_hot_spots_many_rounds(gpu_device, monkeypatch, seed):
     print(seed, levels, (bs, nq, nh, hd, npts), dtype, errs)
 
 
+@pytest.mark.parametrize("rec_lds", [0, 1], ids=["records-one-by-one", "slab-in-LDS"])
+@pytest.mark.parametrize("log2", [8, 7], ids=["tiles-of-256", "tiles-of-128"])
+@pytest.mark.parametrize("seed", range(6))
+def test_finer_tiles_of_the_grad_value_pass(gpu_device, monkeypatch, seed, log2, rec_lds):
+    """The tile pass keeps 32 sums per thread: 512 pixels x 32 channels per workgroup, 256 x 64 or 128 x 128 (one pass
+    over the records for heads of up to 64 / 128 channels, two for more).  The launcher picks the tile size from
+    head_dim and the size of the maps; here both finer sizes are forced on random problems of every head size that is
+    a multiple of four (more sums than channels, exactly as many, two passes), with samples piled on a few spots, tiles
+    split into query chunks or not, float32 and 16-bit storage, and the first kernel's workgroups either storing their
+    records one by one or collecting their slab in LDS."""
+    rng = np.random.default_rng(7000 + seed)
+    env = {"MXD_MSDA_TILE_PX_LOG2": log2, "MXD_MSDA_BWD_REC_LDS": rec_lds}
+    if seed % 2:
+        env["MXD_MSDA_TILE_TARGET"] = 1000000
+    set_tuning(monkeypatch, **env)
+    nl = int(rng.integers(1, 4))
+    levels = [(int(rng.integers(6, 60)), int(rng.integers(6, 60))) for _ in range(nl)]
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh = int(rng.integers(1, 3)), int(rng.integers(1500, 5000)), int(rng.integers(1, 4))
+    hd = int(rng.choice([4, 20, 32, 48, 64, 100, 128, 200, 256]))
+    npts = int(rng.integers(1, 7))
+    dtype = (torch.float32, torch.float16, torch.bfloat16)[seed % 3]
+    g = torch.Generator().manual_seed(7100 + seed)
+    loc = torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.2 - 0.1
+    nspots = int(rng.integers(1, 5))
+    spots = torch.rand(nspots, 2, generator=g) * 1.04 - 0.02
+    pick = torch.randint(0, 3 * nspots + 1, loc.shape[:-1], generator=g)
+    for k in range(nspots):
+        loc[pick == k] = spots[k]
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g), shapes, lsi, loc,
+                               torch.rand(bs, nq, nh, nl, npts, generator=g), torch.randn(bs, nq, nh * hd, generator=g))
+    print("case", seed, levels, (bs, nq, nh, hd, npts), dtype, env, flush=True)
+    if dtype == torch.float32:
+        _check_all(inp, gpu_device, FWD_FP32, BWD_FP32)
+    else:
+        inp = workloads.MsdaInputs(*[t.to(dtype) if t.is_floating_point() else t for t in inp])
+        _check_all(inp, gpu_device, half_tol(dtype), half_tol(dtype))
+
+
 def _random_case(seed):
     """A random small problem: odd sizes everywhere, locations reaching outside the image."""
     rng = np.random.default_rng(seed)
@@ -847,7 +887,8 @@ def test_level_start_indices_that_do_not_tile_the_keys(gpu_device, monkeypatch, 
     """level_start_index is the caller's: the reference's kernels index value with it as given and add gradients with
     atomics, so levels may leave keys uncovered, come in any order or overlap (kernels/multi_scale_deformable_attn/
     op_kernel/multi_scale_deformable_attn_grad.cpp:181-186).  Rows of grad_value that no level covers are exactly zero."""
-    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=cu)
+    # (the forward's form makes no difference to the backward: its runs also take the finest tiles of the grad_value pass)
+    set_tuning(monkeypatch, MXD_MSDA_FWD_CU=cu, MXD_MSDA_TILE_PX_LOG2=7 if cu == "1" else 9)
     levels, starts, nk = _LAYOUTS[layout]
     shapes = torch.tensor(levels, dtype=torch.int64)
     lsi = torch.tensor(starts, dtype=torch.int64)
