@@ -11,7 +11,8 @@ dominant kernel (timed live with HIP events on the launch stream), per-kernel fi
 the CPU oracle timed on the host cores of the same box as a reported baseline.
 Other workloads: the named shapes of drivingsdk_amd.workloads (with --dtype), and the sibling operators
 that run on the same kernels: sparse4d_dagg (deformable aggregation), gka (geometric kernel attention),
-grid_sampler2d (grid_sampler2d_v2), each at a shape of the reference's recipes or tests.
+grid_sampler2d (grid_sampler2d_v2), each at a shape of the reference's recipes or tests; `heuristics` times the
+launcher's default choices against every forced variant on shapes around the benchmark shapes.
 """
 import argparse
 import json
@@ -434,6 +435,117 @@ def _bench_grid_sampler(args):
     print(json.dumps(result))
 
 
+def _bench_heuristics(args):
+    """The launcher's choices against the forms it did not choose, on shapes around the benchmark shapes: for every
+    shape the forward and the backward are timed (raw C-ABI launches, HIP events, the variants taking turns) with the
+    default launch and with each tuning variable forced; the default should be within 5 % of the best.  The table goes
+    to stderr, one JSON line to stdout."""
+    import torch
+
+    from drivingsdk_amd import _lib, workloads
+
+    lib = _lib.load()
+    dev = torch.device("cuda", 0)
+    enc, bev = workloads._DETR_LEVELS, workloads._BEV_LEVELS
+    f32, f16 = torch.float32, torch.float16
+    # name, dtype, bs, queries (None = keys), levels, heads, head_dim, points
+    shapes = [
+        ("encoder", f32, 2, None, enc, 8, 32, 4), ("encoder fp16", f16, 2, None, enc, 8, 32, 4),
+        ("encoder bs1", f32, 1, None, enc, 8, 32, 4), ("encoder bs8", f32, 8, None, enc, 8, 32, 4),
+        ("encoder 4 heads", f32, 2, None, enc, 4, 32, 4), ("encoder 16 heads", f32, 2, None, enc, 16, 32, 4),
+        ("encoder 3 levels", f32, 2, None, enc[:3], 8, 32, 4), ("encoder 5 levels", f32, 2, None, enc + ((7, 10),), 8, 32, 4),
+        ("encoder 6 levels", f32, 2, None, ((200, 300),) + enc + ((7, 10),), 8, 32, 4),
+        ("encoder 2 points", f32, 2, None, enc, 8, 32, 2), ("encoder 8 points", f32, 2, None, enc, 8, 32, 8),
+        ("encoder head_dim 16", f32, 2, None, enc, 8, 16, 4), ("encoder head_dim 64", f32, 2, None, enc, 8, 64, 4),
+        ("encoder head_dim 64 fp16", f16, 2, None, enc, 8, 64, 4), ("encoder head_dim 128 fp16", f16, 1, None, enc, 8, 128, 4),
+        ("decoder 300 queries", f32, 2, 300, enc, 8, 32, 4), ("decoder 900 queries bs8", f32, 8, 900, enc, 8, 32, 4),
+        ("BEVFormer", f32, 6, 9675, bev, 8, 32, 8), ("BEVFormer fp16", f16, 6, 9675, bev, 8, 32, 8),
+        ("BEVFormer 4 points", f32, 6, 9675, bev, 8, 32, 4),
+    ]
+    fwd_variants = [{}, {"MXD_MSDA_FWD_CU": 0}, {"MXD_MSDA_FWD_CU": 1}, {"MXD_MSDA_FWD_CU": 0, "MXD_MSDA_FWD_LDS": 0},
+                    {"MXD_MSDA_FWD_CU": 0, "MXD_MSDA_FWD_LDS": 40960}, {"MXD_MSDA_FWD_CU_FLIP": 0}, {"MXD_MSDA_FWD_CU_FLIP": 1}]
+    bwd_variants = [{}, {"MXD_MSDA_BWD_UNIT_SPLIT": 0}, {"MXD_MSDA_BWD_UNIT_SPLIT": 2}, {"MXD_MSDA_TILE_PX_LOG2": 9}, {"MXD_MSDA_TILE_PX_LOG2": 8},
+                    {"MXD_MSDA_TILE_PX_LOG2": 7}, {"MXD_MSDA_BWD_REC_LDS": 0}, {"MXD_MSDA_BWD_REC_LDS": 1},
+                    {"MXD_MSDA_BWD_LANE_BYTES": 16}, {"MXD_MSDA_BWD_LANE_BYTES": 8}]
+    saved = {k: v for k, v in os.environ.items() if k.startswith("MXD_MSDA_")}
+
+    def set_env(env):
+        for k in [k for k in os.environ if k.startswith("MXD_MSDA_")]:
+            del os.environ[k]
+        for k, v in env.items():
+            os.environ[k] = str(v)
+        _lib.reload_tuning()
+
+    def label(env):
+        return ",".join(f"{k[9:]}={v}" for k, v in env.items()) or "default"
+
+    rows, worst = [], 1.0
+    g = torch.Generator(device=dev).manual_seed(4242)
+    for name, dt, bs, nq, levels, nh, hd, npts in shapes:
+        sh, lsi = workloads.level_tensors(levels)
+        nk, nl = int(sh.prod(1).sum()), len(levels)
+        nq = nk if nq is None else nq
+        code = {f32: 0, f16: 1, torch.bfloat16: 2}[dt]
+        value = torch.randn(bs, nk, nh, hd, device=dev, generator=g).to(dt)
+        ref = torch.rand(bs, nq, 1, 1, 1, 2, device=dev, generator=g)
+        loc = (ref + 0.03 * torch.randn(bs, nq, nh, nl, npts, 2, device=dev, generator=g)).to(dt)
+        attn = torch.softmax(torch.randn(bs, nq, nh, nl * npts, device=dev, generator=g), -1).reshape(bs, nq, nh, nl, npts).to(dt)
+        gout = torch.randn(bs, nq, nh * hd, device=dev, generator=g).to(dt)
+        shd, lsid = sh.int().to(dev), lsi.int().to(dev)
+        out = torch.empty(bs, nq, nh * hd, dtype=dt, device=dev)
+        gv, gl, ga = torch.empty_like(value), torch.empty_like(loc), torch.empty_like(attn)
+        dims = (bs, nk, nh, hd, nl, nl, nq, npts)
+        set_env({"MXD_MSDA_TILE_PX_LOG2": 7, "MXD_MSDA_BWD_REC_LDS": 1})   # (the largest workspace any variant needs)
+        ws_bytes = max(lib.mxd_msda_backward_workspace_bytes(code, *dims), 16)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def fwd():
+            rc = lib.mxd_msda_forward(value.data_ptr(), shd.data_ptr(), lsid.data_ptr(), loc.data_ptr(), attn.data_ptr(),
+                                      out.data_ptr(), code, *dims, stream)
+            assert rc == 0, _lib.last_error()
+
+        def bwd():
+            rc = lib.mxd_msda_backward(value.data_ptr(), shd.data_ptr(), lsid.data_ptr(), loc.data_ptr(), attn.data_ptr(),
+                                       gout.data_ptr(), gv.data_ptr(), gl.data_ptr(), ga.data_ptr(), ws.data_ptr(), ws_bytes,
+                                       code, *dims, 0, stream)
+            assert rc == 0, _lib.last_error()
+
+        samples = bs * nq * nh * nl * npts
+        iters = max(10, min(100, int(3e8 / samples)))
+        for what, fn, variants in (("forward", fwd, fwd_variants), ("backward", bwd, bwd_variants)):
+            times, same = {}, {}
+            # variants whose plan equals the default's are the default: skip them
+            set_env({})
+            plan0 = _lib.make_plan(what == "backward", code, *dims).as_dict()
+            for rep in range(2):
+                for env in variants:
+                    set_env(env)
+                    if env and rep == 0:
+                        same[label(env)] = _lib.make_plan(what == "backward", code, *dims).as_dict() == plan0 and \
+                            not any(k in env for k in ("MXD_MSDA_FWD_CU_FLIP", "MXD_MSDA_TILE_PX_LOG2", "MXD_MSDA_BWD_REC_LDS",
+                                                       "MXD_MSDA_BWD_UNIT_SPLIT"))
+                    if same.get(label(env)):
+                        continue
+                    t = _event_ms(fn, iters, iters) * 1e3
+                    times[label(env)] = min(times.get(label(env), 1e30), t)
+            best = min(times, key=times.get)
+            # (launches of a few microseconds differ by more than 5 % from run to run: a microsecond is allowed)
+            ratio = 1.0 if times["default"] - times[best] <= 1.0 else times["default"] / times[best]
+            worst = max(worst, ratio)
+            rows.append({"shape": name, "pass": what, "default_us": times["default"], "best": best, "best_us": times[best],
+                         "default_over_best": ratio, "us": times})
+            print(f"{name:28s} {what:8s} default {times['default']:8.1f} us  best {best:28s} {times[best]:8.1f} us  "
+                  f"ratio {ratio:5.3f}  " + "  ".join(f"{k}={v:.1f}" for k, v in times.items() if k != "default"),
+                  file=sys.stderr, flush=True)
+        del value, loc, attn, gout, out, gv, gl, ga, ws
+    set_env(saved)
+    print(json.dumps({"metric": "launch heuristics: time of the default launch over the best forced variant, worst shape",
+                      "value": worst, "unit": "ratio", "n_gpus": 1, "higher_is_better": False, "data": "synthetic",
+                      "config": {"workload": "heuristics: forward and backward of %d shapes around the benchmark shapes" % len(shapes)},
+                      "all_within_5pct": worst <= 1.05, "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -467,6 +579,8 @@ def main():
         return _bench_gka(args)
     if args.workload == "grid_sampler2d":
         return _bench_grid_sampler(args)
+    if args.workload == "heuristics":
+        return _bench_heuristics(args)
     dev = torch.device("cuda", 0)
     dtype = getattr(torch, args.dtype)
     inp = workloads.make_inputs(args.workload, dtype=dtype, with_grad_output=True)

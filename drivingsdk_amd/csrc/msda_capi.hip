@@ -85,7 +85,8 @@ struct Tuning {
     int tile_order;      // MXD_MSDA_TILE_ORDER: 1 = work items of the tile pass batch-major, 0 = item-major, -1 = chosen here
     int bwd_sparse;      // MXD_MSDA_BWD_SPARSE: 0 = zero-fill (and, for 16-bit dtypes, round) the whole fp32 image of
                          // grad_value, 1 = only the rows that receive atomic additions
-    int bwd_unit_split;  // MXD_MSDA_BWD_UNIT_SPLIT: 0 = a unit of the first backward kernel is always a whole query
+    int bwd_unit_split;  // MXD_MSDA_BWD_UNIT_SPLIT: 0 = a unit of the first backward kernel is always a whole query, 1 = queries
+                         // of 25 to 32 samples get two units, 2 = queries of 17 to 32 samples
     int bwd_lane_bytes;  // MXD_MSDA_BWD_LANE_BYTES: most bytes of a row one lane of the first backward kernel loads
                          // (16, 8, 4), 0 = chosen here
     int tile_px_log2;    // MXD_MSDA_TILE_PX_LOG2: log2 of the pixels per tile of the grad_value pass (9, 8, 7), 0 = chosen here
@@ -288,8 +289,12 @@ static int64_t bwd_tile_q(int dtype, const Dims& d)
     // 16 of its samples, so that the workgroup -- half as many queries -- stages all its samples while it counts its
     // records (their geometry is derived once) and collects its records in LDS to write its slab in whole lines, as
     // with up to 16 samples per query.
+    // (it pays when the second unit has work for most of its lanes -- encoder levels, float32: 32 samples per query 544
+    //  against 571 us, BEVFormer 1036 against 1094; 24 samples 2370 against 2301, 20 samples 442 against 420 --: from 25
+    //  samples on; MXD_MSDA_BWD_UNIT_SPLIT=2 splits from 17 on)
     const int units = mxd::kWave / lpr * 4;
-    if (tuning().bwd_unit_split && least == units && units >= 8 && d.nl * d.np > mxd::kChunk && d.nl * d.np <= 2 * mxd::kChunk)
+    const int64_t split_from = tuning().bwd_unit_split >= 2 ? mxd::kChunk + 1 : mxd::kChunk + mxd::kChunk / 2 + 1;
+    if (tuning().bwd_unit_split && least == units && units >= 8 && d.nl * d.np >= split_from && d.nl * d.np <= 2 * mxd::kChunk)
         return least / 2;
     return least;
 }
@@ -379,11 +384,14 @@ size_t bwd_workspace_bytes(int dtype, const Dims& d)
 int plan_record_buffer(mxd_msda_plan* p, const BwdLayout& L, const Dims& d, int dtype, bool plain_or_fused, int unit_split_log2)
 {
     if (!L.tiles) return 0;
-    // By default for 16-bit rows only (MXD_MSDA_BWD_REC_LDS=1: wherever it fits).  Measured, backward at 8 heads x 128
-    // channels with tiles of 128 pixels: float16 414 -> 383 us; float32 586 -> 596 us, geometric kernel attention (64
-    // channels, float32) 0.80 -> 0.86 ms per step -- there the buffer costs the kernel a workgroup per CU, which weighs
-    // more than the partial lines.
-    if (tuning().bwd_rec_lds < 0 && elem_size(dtype) != 2) return 0;
+    // By default for the plain operator and its fused form, for slabs of up to 12 KiB and, with 16-bit rows, of up to
+    // 24 KiB (MXD_MSDA_BWD_REC_LDS=1: wherever it fits).  Measured, backward: encoder levels with 2 points, float32 (12 KiB)
+    // 231 -> 216 us; 8 heads x 128 channels, tiles of 128 pixels (24 KiB): float16 414 -> 383 us, float32 586 -> 596 us;
+    // geometric kernel attention (64 channels, float32, 23 KiB) 0.80 -> 0.86 ms per step -- where it loses the buffer
+    // costs the kernel a workgroup per CU, which weighs more than the partial lines.
+    if (tuning().bwd_rec_lds < 0 &&
+        !(plain_or_fused && L.rec_cap * (mxd::kRecDwords * 4) <= (elem_size(dtype) == 2 ? 24 : 12) * 1024))
+        return 0;
     const bool one_pass = plain_or_fused && p->iters == 1 && d.nl * d.np <= ((int64_t)mxd::kChunk << unit_split_log2);
     const int64_t bytes = L.rec_cap * (mxd::kRecDwords * 4);
     const int64_t total = (((int64_t)p->lds_bytes + 15) & ~(int64_t)15) + bytes;
@@ -579,7 +587,9 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
         // outweigh the gain.  Measured at the encoder shape with the 16 (batch, head) pairs split as bs x heads --
         // this form against the general kernel: 2 x 8: 91 / 102 us, 1 x 16: 96 / 123, 4 x 4: 102 / 102, 8 x 2: 120 / 105
         // (152 with one round of workgroups), 16 x 1: 133 / 112 (175), 2 x 6 heads, no pinning: 106 / 94.
-        if (mode < 0 && (trial.xcd_mode != 1 || trial.heads_per_xcd > 2)) continue;
+        // (four heads, each shared by two XCDs: with the encoder's queries and two batch elements 44.8 against 50.2 us)
+        if (mode < 0 && !((trial.xcd_mode == 1 && trial.heads_per_xcd <= 2) || (trial.xcd_mode == 2 && trial.xcds_per_head <= 2)))
+            continue;
         double over = ceil(slices) * slice_bytes / (4.0 * 1024 * 1024) - 0.4;
         over = over < 0.0 ? 0.0 : (over > 1.0 ? 1.0 : over);
         const double gather = (1.0 + 0.5 * over) * (double)tq * (double)(d.nl * d.np) * 4.0;

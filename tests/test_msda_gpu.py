@@ -504,12 +504,13 @@ def test_backward_launch_variants_agree_with_the_oracle(gpu_device, monkeypatch,
         print(env, name, errs)
 
 
-@pytest.mark.parametrize("split", ["1", "0"], ids=["two-units-per-query", "one-unit-per-query"])
+@pytest.mark.parametrize("split", ["2", "0"], ids=["two-units-per-query", "one-unit-per-query"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("nl,nl_attn,npts", [(4, 4, 8), (3, 3, 7), (2, 3, 12), (1, 1, 17), (4, 5, 5)])
 def test_queries_of_17_to_32_samples(gpu_device, monkeypatch, nl, nl_attn, npts, dtype, split):
-    """The backward's first kernel gives a query of 17 to 32 samples two units of 16 samples each (workgroups of half as
-    many queries that make one pass); MXD_MSDA_BWD_UNIT_SPLIT=0 keeps one unit per query and two chunks.  Both against
+    """The backward's first kernel can give a query of 17 to 32 samples two units of 16 samples each (workgroups of half
+    as many queries that make one pass: by default from 25 samples on, with MXD_MSDA_BWD_UNIT_SPLIT=2 from 17 on);
+    MXD_MSDA_BWD_UNIT_SPLIT=0 keeps one unit per query and two chunks.  Both against
     the oracle, with a query count that leaves the last workgroup partly filled and, in two cases, level slots in the
     weights beyond spatial_shapes (zero gradients)."""
     set_tuning(monkeypatch, MXD_MSDA_BWD_UNIT_SPLIT=split)
@@ -524,7 +525,7 @@ def test_queries_of_17_to_32_samples(gpu_device, monkeypatch, nl, nl_attn, npts,
                                torch.randn(bs, nq, nh * hd, generator=g).to(dtype))
     plan = _lib.make_plan(1, {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype], bs, nk, nh, hd, nl, nl_attn, nq, npts)
     units = plan.units_per_wave * plan.waves_per_block * plan.iters
-    assert plan.tile_q * (2 if split == "1" else 1) == units
+    assert plan.tile_q * (2 if split == "2" else 1) == units
     tol = (FWD_FP32, BWD_FP32) if dtype == torch.float32 else (half_tol(dtype),) * 2
     errs = _check_all(inp, gpu_device, *tol)
     if nl_attn > nl:
