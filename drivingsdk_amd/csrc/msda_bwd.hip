@@ -885,8 +885,12 @@ static hipError_t launch_dtype(const KArgs& a, bool scatter, hipStream_t stream)
     if (vec == 2 && np == 1) return launch_one<T, 2, 1>(a, scatter, stream);
     if (vec == 2 && np == 2) return launch_one<T, 2, 2>(a, scatter, stream);
     if (vec == 4 && np == 1) return launch_one<T, 4, 1>(a, scatter, stream);
+    if constexpr (sizeof(T) == 4) {
+        if (vec == 4 && np == 2) return launch_one<T, 4, 2>(a, scatter, stream);
+    }
     if constexpr (sizeof(T) == 2) {
         if (vec == 8 && np == 1) return launch_one<T, 8, 1>(a, scatter, stream);
+        if (vec == 8 && np == 2) return launch_one<T, 8, 2>(a, scatter, stream);
     }
     return hipErrorInvalidConfiguration;
 }

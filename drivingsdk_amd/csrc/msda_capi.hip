@@ -90,6 +90,8 @@ struct Tuning {
     int bwd_lane_bytes;  // MXD_MSDA_BWD_LANE_BYTES: most bytes of a row one lane of the first backward kernel loads
                          // (16, 8, 4), 0 = chosen here
     int tile_px_log2;    // MXD_MSDA_TILE_PX_LOG2: log2 of the pixels per tile of the grad_value pass (9, 8, 7), 0 = chosen here
+    int bwd_two_pass;    // MXD_MSDA_BWD_TWO_PASS: 1 = the first backward kernel reads rows of 17 to 32 lanes of 16 bytes with 16
+                         // lanes in two passes, 0 = with 32 lanes in one
     int bwd_rec_lds;     // MXD_MSDA_BWD_REC_LDS: 0 = workgroups of the first backward kernel that make several passes store
                          // their records one by one, 1 = they collect their slab in LDS wherever it fits, -1 = chosen here
 };
@@ -117,6 +119,7 @@ void read_tuning()
     t.bwd_unit_split = env_int("MXD_MSDA_BWD_UNIT_SPLIT", 1);
     t.tile_px_log2 = env_int("MXD_MSDA_TILE_PX_LOG2", 0);
     t.bwd_rec_lds = env_int("MXD_MSDA_BWD_REC_LDS", -1);
+    t.bwd_two_pass = env_int("MXD_MSDA_BWD_TWO_PASS", 1);
     g_tuning = t;
 }
 
@@ -232,7 +235,10 @@ size_t backward_lds_bytes(int units_per_wave, int waves, bool tiles, int64_t tbl
 }
 
 // Row geometry of a problem: elements per lane, lanes per row, row passes.
-void row_geometry(int es, int64_t hd, int align_bytes, int* vec_out, int* lpr_out, int* npass_out)
+// two_pass_rows: rows of 17 to 32 lanes of 16 bytes are read by 16 lanes in two passes instead (four units per
+// wavefront rather than two: the first backward kernel then fills its geometry lanes and sums its dots over 16 lanes
+// with DPP alone; backward at 8 heads x 128 channels in float32 587 -> 572 us, 545 with the slab collected in LDS).
+void row_geometry(int es, int64_t hd, int align_bytes, int* vec_out, int* lpr_out, int* npass_out, bool two_pass_rows = false)
 {
     if (align_bytes < es) align_bytes = es;
     int vec = 16 / es;
@@ -240,6 +246,7 @@ void row_geometry(int es, int64_t hd, int align_bytes, int* vec_out, int* lpr_ou
     const int lanes_needed = (int)((hd + vec - 1) / vec);
     int lpr = 4;
     while (lpr < lanes_needed && lpr < mxd::kWave) lpr <<= 1;
+    if (two_pass_rows && vec * es == 16 && lpr == 32) lpr = 16;
     int npass = (lanes_needed + lpr - 1) / lpr;
     if (npass == 3) npass = 4;
     *vec_out = vec;
@@ -272,7 +279,7 @@ static int64_t bwd_tile_q(int dtype, const Dims& d)
 {
     // (units with very many samples -- deformable aggregation's 312 -- measured 1 to 2 % better with 64)
     int vec, lpr, npass;
-    row_geometry(elem_size(dtype), d.hd, backward_lane_bytes(dtype, d), &vec, &lpr, &npass);
+    row_geometry(elem_size(dtype), d.hd, backward_lane_bytes(dtype, d), &vec, &lpr, &npass, tuning().bwd_two_pass != 0);
     const int64_t least = (mxd::kWave / lpr > 8 || d.nl * d.np >= 256) ? 64 : 32;
     const int v = tuning().bwd_tile_q;
     if (v == 32 || v == 64 || v == 128 || v == 256) return v < least ? least : v;
@@ -343,7 +350,7 @@ BwdLayout bwd_layout_for(int dtype, const Dims& d, int tile_px_log2)
     const int64_t tbl = d.bs * d.nh * L.nwg * L.tbl_stride * 4;
     // dynamic LDS of the first kernel with the most units per wavefront the row can have (16-byte aligned pointers)
     int vec, lpr, npass;
-    row_geometry(elem_size(dtype), d.hd, backward_lane_bytes(dtype, d), &vec, &lpr, &npass);
+    row_geometry(elem_size(dtype), d.hd, backward_lane_bytes(dtype, d), &vec, &lpr, &npass, tuning().bwd_two_pass != 0);
     const size_t lds = backward_lds_bytes(mxd::kWave / lpr, 4, true, L.tbl_stride);
     L.tiles = tuning().bwd_atomic == 0 &&
               L.tbl_stride <= 4096 &&                      // counters of the first kernel live in LDS ...
@@ -384,14 +391,15 @@ size_t bwd_workspace_bytes(int dtype, const Dims& d)
 int plan_record_buffer(mxd_msda_plan* p, const BwdLayout& L, const Dims& d, int dtype, bool plain_or_fused, int unit_split_log2)
 {
     if (!L.tiles) return 0;
-    // By default for the plain operator and its fused form, for slabs of up to 12 KiB and, with 16-bit rows, of up to
-    // 24 KiB (MXD_MSDA_BWD_REC_LDS=1: wherever it fits).  Measured, backward: encoder levels with 2 points, float32 (12 KiB)
-    // 231 -> 216 us; 8 heads x 128 channels, tiles of 128 pixels (24 KiB): float16 414 -> 383 us, float32 586 -> 596 us;
-    // geometric kernel attention (64 channels, float32, 23 KiB) 0.80 -> 0.86 ms per step -- where it loses the buffer
-    // costs the kernel a workgroup per CU, which weighs more than the partial lines.
-    if (tuning().bwd_rec_lds < 0 &&
-        !(plain_or_fused && L.rec_cap * (mxd::kRecDwords * 4) <= (elem_size(dtype) == 2 ? 24 : 12) * 1024))
-        return 0;
+    // By default for the plain operator and its fused form, for slabs of up to 12 KiB and, with at most four units per
+    // wavefront (rows of 16 lanes and more, whose staging strips are small), of up to 24 KiB (MXD_MSDA_BWD_REC_LDS=1:
+    // wherever it fits).  Measured, backward: encoder levels with 2 points, float32 (12 KiB) 231 -> 216 us; 8 heads x 128
+    // channels, tiles of 128 pixels (24 KiB, four units): float16 414 -> 383 us, float32 572 -> 545 us (with two units of
+    // 32 lanes: 586 -> 596); geometric kernel attention (64 channels, float32, 23 KiB) 0.80 -> 0.86 ms per step -- where
+    // it loses, the buffer costs the kernel a workgroup per CU, which weighs more than the partial lines.
+    (void)dtype;
+    const int64_t slab = L.rec_cap * (mxd::kRecDwords * 4);
+    if (tuning().bwd_rec_lds < 0 && !(plain_or_fused && (slab <= 12 * 1024 || p->units_per_wave <= 4))) return 0;
     const bool one_pass = plain_or_fused && p->iters == 1 && d.nl * d.np <= ((int64_t)mxd::kChunk << unit_split_log2);
     const int64_t bytes = L.rec_cap * (mxd::kRecDwords * 4);
     const int64_t total = (((int64_t)p->lds_bytes + 15) & ~(int64_t)15) + bytes;
@@ -639,7 +647,8 @@ int make_plan(int backward, int dtype, const Dims& d, int align_bytes, mxd_msda_
     const int es = elem_size(dtype);
     int vec, lpr, npass;
     if (backward && align_bytes > backward_lane_bytes(dtype, d)) align_bytes = backward_lane_bytes(dtype, d);
-    row_geometry(es, d.hd, align_bytes, &vec, &lpr, &npass);
+    // (the forward keeps 32 lanes in one pass: at 8 heads x 128 channels in float32 two passes take 248 against 237 us)
+    row_geometry(es, d.hd, align_bytes, &vec, &lpr, &npass, backward && tuning().bwd_two_pass != 0);
     if (!backward && cu_form && *cu_form && level_cache) {
         if (plan_forward_cu(dtype, d, vec, lpr, npass, p, level_cache)) return MXD_OK;
     }

@@ -185,11 +185,12 @@ size_t mxd_msda_backward_workspace_bytes(int dtype, int64_t bs, int64_t nk, int6
                                 form of the backward: the levels may leave keys uncovered, come in any order and
                                 overlap, as for the reference's atomic-add kernel
                                 (op_kernel/multi_scale_deformable_attn_grad.cpp:181-186).  One case is slow by default:
-                                levels that overlap so far that they have more than num_keys/512 + num_levels tiles of
-                                512 pixels between them -- mxd_msda_backward then adds the levels beyond that sample
-                                by sample.  The fused form and the sibling operators have no such fallback: there the
-                                default form leaves those levels out of grad_value, and this flag (or
-                                MXD_MSDA_BWD_ATOMIC=1 in the environment) asks for the form that does not care */
+                                levels that overlap so far that they have more than num_keys/T + num_levels tiles of
+                                T pixels between them (T = 512 for heads of up to 32 channels, 256 for up to 64, 128
+                                beyond) -- mxd_msda_backward then adds the levels beyond that sample by sample.  The
+                                fused form and the sibling operators have no such fallback: there the default form
+                                leaves those levels out of grad_value, and this flag (or MXD_MSDA_BWD_ATOMIC=1 in the
+                                environment) asks for the form that does not care */
 
 /* Backward.  Replaces multi_scale_deformable_attn_backward
  * (mx_driving/csrc/MultiScaleDeformableAttn.cpp:68-118).  On `hip_stream`, in order:

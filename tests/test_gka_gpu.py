@@ -7,7 +7,7 @@ import torch
 import mx_driving
 from drivingsdk_amd import _lib
 from oracle import gka_oracle as gka
-from util import BWD_FP32, FWD_FP32, HALF, rel_err
+from util import BWD_FP32, FWD_FP32, HALF, rel_err, set_tuning
 
 pytestmark = pytest.mark.gpu
 
@@ -117,3 +117,28 @@ def test_largest_reference_shape_at_full_batch(gpu_device):
     got = run_gpu(*inp, gpu_device)
     for name, g_, w_, tol in zip(("output", "grad_value", "grad_attn_weights"), got, want, (FWD_FP32, BWD_FP32, BWD_FP32)):
         assert rel_err(g_, w_) <= tol, (name, rel_err(g_, w_))
+
+
+def test_levels_that_overlap_beyond_the_run_table_take_the_atomic_form(gpu_device, monkeypatch):
+    """level_start_index is the caller's.  Three levels of 513 pixels that overlap inside 600 keys have six tiles of 512
+    pixels between them where the run table of the tile-mode backward has room for four (num_keys / 512 + num_levels).
+    The plain operator adds such levels sample by sample; this operator documents that its default form leaves them out
+    of grad_value and that MXD_MSDA_BWD_ATOMIC=1 (the one-kernel form with global atomics) takes any layout: that form
+    must give the oracle's gradients, and the forward and grad_attn_weights must not depend on the form."""
+    bs, nq, hd, nh, nl, npts, hw = 2, 400, 16, 3, 3, 5, (27, 19)
+    g = torch.Generator().manual_seed(513)
+    sh = torch.tensor([list(hw)] * nl)
+    lsi = torch.tensor([0, 40, 87])
+    nk = 600
+    loc = torch.stack((torch.randint(-2, hw[1] + 2, (bs, nq, nh, nl, npts), generator=g),
+                       torch.randint(-2, hw[0] + 2, (bs, nq, nh, nl, npts), generator=g)), -1).float()
+    value = torch.rand(bs, nk, nh, hd, generator=g) * 3
+    attn = torch.rand(bs, nq, nh, nl, npts, generator=g)
+    go = torch.rand(bs, nq, nh * hd, generator=g) * 10
+    want = (gka.forward(value, sh, lsi, loc, attn),) + gka.backward(value, sh, lsi, loc, attn, go)
+    default = run_gpu(value, sh, lsi, loc, attn, go, gpu_device)
+    set_tuning(monkeypatch, MXD_MSDA_BWD_ATOMIC=1)
+    got = run_gpu(value, sh, lsi, loc, attn, go, gpu_device)
+    for name, g_, w_, tol in zip(("output", "grad_value", "grad_attn_weights"), got, want, (FWD_FP32, BWD_FP32, BWD_FP32)):
+        assert rel_err(g_, w_) <= tol, (name, rel_err(g_, w_))
+    assert rel_err(default[0], want[0]) <= FWD_FP32 and rel_err(default[2], want[2]) <= BWD_FP32
