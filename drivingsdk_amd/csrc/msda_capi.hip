@@ -78,6 +78,8 @@ struct Tuning {
     int fwd_cu;          // MXD_MSDA_FWD_CU: 0 = never use the one-workgroup-per-CU forward, 1 = whenever it can run,
                          // -1 = for problems large enough to pay for it
     int fwd_cu_wgs;      // MXD_MSDA_FWD_CU_WGS: its workgroups per (batch, head), 0 = chosen here
+    int fwd_cu_cache;    // MXD_MSDA_FWD_CU_CACHE: most bytes of LDS its level cache takes, -1 = all the CU has (a small value
+                         // makes every sample come from memory: a hook for measurements)
     int fwd_cu_flip;     // MXD_MSDA_FWD_CU_FLIP: 1 = half of its wavefronts gather from LDS first, the others from memory
                          // first; 0 = all in the same order (sums then formed in the general kernel's order, bit for bit);
                          // -1 = chosen here
@@ -112,6 +114,7 @@ void read_tuning()
     t.fwd_cu = env_int("MXD_MSDA_FWD_CU", -1);
     t.fwd_cu_wgs = env_int("MXD_MSDA_FWD_CU_WGS", 0);
     t.fwd_cu_flip = env_int("MXD_MSDA_FWD_CU_FLIP", -1);
+    t.fwd_cu_cache = env_int("MXD_MSDA_FWD_CU_CACHE", -1);
     t.bwd_fill_kernel = env_int("MXD_MSDA_BWD_FILL_KERNEL", 0);
     t.tile_order = env_int("MXD_MSDA_TILE_ORDER", -1);
     t.bwd_lane_bytes = env_int("MXD_MSDA_BWD_LANE_BYTES", 0);
@@ -624,6 +627,11 @@ bool plan_forward_cu(int dtype, const Dims& d, int vec, int lpr, int npass, mxd_
     p->block = (uint32_t)(mxd::kCuWaves * mxd::kWave);
     p->lds_bytes = (uint32_t)mxd::kCuLdsBytes;
     *cache_bytes = cap & ~15;
+    if (tuning().fwd_cu_cache >= 0 && tuning().fwd_cu_cache < *cache_bytes) {
+        // (at least the row of zeros that stands for corners outside the image)
+        const int least = (int)(d.hd * es + 15) & ~15;
+        *cache_bytes = tuning().fwd_cu_cache < least ? least : (tuning().fwd_cu_cache & ~15);
+    }
     return true;
 }
 

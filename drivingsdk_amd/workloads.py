@@ -28,6 +28,10 @@ WORKLOADS = {
     "bevformer_sca": dict(bs=6, nq=9675, levels=_BEV_LEVELS, nh=8, hd=32, np=8, loc="anchor_cluster", seed=1003),
     "head_dim_128": dict(bs=1, nq=None, levels=_DETR_LEVELS, nh=8, hd=128, np=4, loc="uniform", seed=1004),
     "detr_encoder_bwd": dict(bs=2, nq=None, levels=_DETR_LEVELS, nh=8, hd=32, np=4, loc="ref_plus_offset", seed=1005),
+    # the encoder's queries over its two coarse levels only, 8 points each (16 samples per query as in the encoder): every
+    # row fits the LDS of a CU, so the forward's one-workgroup-per-CU form gathers nothing from memory -- the
+    # measurement twin of the encoder shape with MXD_MSDA_FWD_CU_CACHE=0 (everything from memory)
+    "detr_encoder_coarse": dict(bs=2, nq=19947, levels=_DETR_LEVELS[2:], nh=8, hd=32, np=8, loc="ref_plus_offset", seed=1006),
 }
 
 
