@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define MXD_MSDA_VERSION 102 /* major*10000 + minor*100 + patch */
+#define MXD_MSDA_VERSION 103 /* major*10000 + minor*100 + patch */
 
 /* dtype codes */
 #define MXD_DTYPE_F32 0

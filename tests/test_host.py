@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.mxd_msda_version() == 102
+    assert lib.mxd_msda_version() == 103
 
 
 def test_public_names_match_the_reference_module():
@@ -293,7 +293,7 @@ def test_header_compiles_as_c99_and_the_library_links(tmp_path):
                     "-Wl,-rpath,/opt/rocm/lib"], check=True, capture_output=True, text=True)
     res = subprocess.run([str(exe)], capture_output=True, text=True)
     assert res.returncode == 0, (res.returncode, res.stdout, res.stderr)
-    assert res.stdout.startswith("ok 102")
+    assert res.stdout.startswith("ok 103")
 
 
 def test_backward_runs_every_fallible_step_before_its_first_launch(monkeypatch):

@@ -80,7 +80,7 @@ def _check_all(inp, device, fwd_tol, bwd_tol, with_grads=True):
 
 def test_library_is_the_in_tree_build():
     lib = _lib.load()
-    assert lib.mxd_msda_version() == 102
+    assert lib.mxd_msda_version() == 103
     with open("/proc/self/maps") as f:
         assert any("drivingsdk_amd/lib/libmxd_msda.so" in line for line in f)
 
