@@ -36,9 +36,13 @@
 
 namespace mxd {
 
-template <typename T, int VEC, int NPASS, bool SCATTER, int SRC>
+// RECBUF: workgroups that make several passes collect their slab of records in LDS (see `recbuf` below); an
+// instantiation of its own, for the plain operator and its fused form, because the extra paths cost the others scalar
+// registers (spilled ones travel through vector lanes) that they have no use for.
+template <typename T, int VEC, int NPASS, bool SCATTER, int SRC, bool RECBUF = false>
 __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
+    static_assert(!RECBUF || (!SCATTER && (SRC == kSrcPlain || SRC == kSrcFused)), "the record buffer is built for the tile form of the operator and its fused form");
     constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
     constexpr bool FUSED = SRC == kSrcFused;
     constexpr int NC = SRC == kSrcGka ? 1 : 4;  // corner rows per sample (geometric kernel attention: one pixel)
@@ -414,7 +418,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     // shorter, the smaller the tiles of the grad_value pass are -- reach memory as partial lines.
     typedef uint32_t __attribute__((may_alias)) u32_alias;
     u32_alias* recbuf = nullptr;
-    if constexpr (!SCATTER) {
+    if constexpr (RECBUF) {
         if (!rec_in_lds && a.rec_lds_bytes != 0)
             recbuf = reinterpret_cast<u32_alias*>(smem + ((reinterpret_cast<unsigned char*>(cursor + a.tbl_stride) - smem + 15) & ~(size_t)15));
     }
@@ -671,7 +675,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                                                __builtin_bit_cast(uint32_t, rec_wa[r]), __builtin_bit_cast(uint32_t, rec_wb[r]), 0u};
                             if (rec_in_lds) {
                                 *rec_lds(pos) = rec;
-                            } else if (recbuf != nullptr) {
+                            } else if (RECBUF && recbuf != nullptr) {
                                 recbuf[3 * pos] = rec.x;
                                 recbuf[3 * pos + 1] = rec.y;
                                 recbuf[3 * pos + 2] = rec.z;
@@ -703,7 +707,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             }
         }
     }
-    if constexpr (!SCATTER) {
+    if constexpr (RECBUF) {
         if (recbuf != nullptr) {  // (uniform over the workgroup; every wavefront leaves the loop above)
             __syncthreads();
             // the slab as it lies in the buffer: 16 bytes per lane, then the odd words
@@ -864,11 +868,15 @@ static hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
     } else if (a.ref != nullptr) {
         if (scatter)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcFused>), grid, block, a.plan.lds_bytes, stream, a);
+        else if (a.rec_lds_bytes != 0)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcFused, true>), grid, block, a.plan.lds_bytes, stream, a);
         else
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcFused>), grid, block, a.plan.lds_bytes, stream, a);
     } else {
         if (scatter)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcPlain>), grid, block, a.plan.lds_bytes, stream, a);
+        else if (a.rec_lds_bytes != 0)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcPlain, true>), grid, block, a.plan.lds_bytes, stream, a);
         else
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcPlain>), grid, block, a.plan.lds_bytes, stream, a);
     }

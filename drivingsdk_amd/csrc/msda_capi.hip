@@ -393,7 +393,7 @@ size_t bwd_workspace_bytes(int dtype, const Dims& d)
 // fused form) collects its records in its staging strips instead.  Adds the bytes to the plan.
 int plan_record_buffer(mxd_msda_plan* p, const BwdLayout& L, const Dims& d, int dtype, bool plain_or_fused, int unit_split_log2)
 {
-    if (!L.tiles) return 0;
+    if (!L.tiles || !plain_or_fused) return 0;  // (the kernel is built with the buffer for these two sources only)
     // By default for the plain operator and its fused form, for slabs of up to 12 KiB and, with at most four units per
     // wavefront (rows of 16 lanes and more, whose staging strips are small), of up to 24 KiB (MXD_MSDA_BWD_REC_LDS=1:
     // wherever it fits).  Measured, backward: encoder levels with 2 points, float32 (12 KiB) 231 -> 216 us; 8 heads x 128
@@ -402,7 +402,7 @@ int plan_record_buffer(mxd_msda_plan* p, const BwdLayout& L, const Dims& d, int 
     // it loses, the buffer costs the kernel a workgroup per CU, which weighs more than the partial lines.
     (void)dtype;
     const int64_t slab = L.rec_cap * (mxd::kRecDwords * 4);
-    if (tuning().bwd_rec_lds < 0 && !(plain_or_fused && (slab <= 12 * 1024 || p->units_per_wave <= 4))) return 0;
+    if (tuning().bwd_rec_lds < 0 && !(slab <= 12 * 1024 || p->units_per_wave <= 4)) return 0;
     const bool one_pass = plain_or_fused && p->iters == 1 && d.nl * d.np <= ((int64_t)mxd::kChunk << unit_split_log2);
     const int64_t bytes = L.rec_cap * (mxd::kRecDwords * 4);
     const int64_t total = (((int64_t)p->lds_bytes + 15) & ~(int64_t)15) + bytes;
