@@ -92,6 +92,8 @@ struct Tuning {
     int bwd_lane_bytes;  // MXD_MSDA_BWD_LANE_BYTES: most bytes of a row one lane of the first backward kernel loads
                          // (16, 8, 4), 0 = chosen here
     int tile_px_log2;    // MXD_MSDA_TILE_PX_LOG2: log2 of the pixels per tile of the grad_value pass (9, 8, 7), 0 = chosen here
+    int bwd_fixed;       // MXD_MSDA_BWD_FIXED: 0 = the first backward kernel never takes the instantiation with the common launch
+                         // geometry as constants (default 1: where the launch has that geometry)
     int bwd_two_pass;    // MXD_MSDA_BWD_TWO_PASS: 1 = the first backward kernel reads rows of 17 to 32 lanes of 16 bytes with 16
                          // lanes in two passes, 0 = with 32 lanes in one
     int bwd_rec_lds;     // MXD_MSDA_BWD_REC_LDS: 0 = workgroups of the first backward kernel that make several passes store
@@ -122,6 +124,7 @@ void read_tuning()
     t.bwd_unit_split = env_int("MXD_MSDA_BWD_UNIT_SPLIT", 1);
     t.tile_px_log2 = env_int("MXD_MSDA_TILE_PX_LOG2", 0);
     t.bwd_rec_lds = env_int("MXD_MSDA_BWD_REC_LDS", -1);
+    t.bwd_fixed = env_int("MXD_MSDA_BWD_FIXED", 1);
     t.bwd_two_pass = env_int("MXD_MSDA_BWD_TWO_PASS", 1);
     g_tuning = t;
 }
@@ -1024,6 +1027,10 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     a.tile_px_log2 = L.tile_px_log2;
     a.unit_split_log2 = unit_split_log2(a.plan);
     a.rec_lds_bytes = plan_record_buffer(&a.plan, L, d, dtype, !gka && !grid, a.unit_split_log2);
+    a.bwd_fixed = (tuning().bwd_fixed != 0 && !fused && !gka && !grid && L.tiles && a.plan.lanes_per_row == 8 && a.plan.units_per_wave == 8 &&
+                   a.plan.npass == 1 && a.plan.iters == 1 && a.unit_split_log2 <= 1 &&
+                   d.nl * d.np <= ((int64_t)mxd::kChunk << a.unit_split_log2) && a.rec_lds_bytes == 0)
+                      ? 1 + a.unit_split_log2 : 0;
     a.meta_i64 = meta64;
     a.value = value;
     a.shapes = spatial_shapes;

@@ -534,6 +534,34 @@ def test_queries_of_17_to_32_samples(gpu_device, monkeypatch, nl, nl_attn, npts,
     print(errs)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("nl,npts", [(4, 4), (3, 5), (1, 1), (4, 8), (2, 13)])
+def test_first_backward_kernel_with_its_geometry_as_constants(gpu_device, monkeypatch, nl, npts, dtype):
+    """Launches whose rows are read by 8 lanes and whose workgroups make one pass (up to 16 samples per query, or up to 32
+    with two units per query) take an instantiation of the first backward kernel that has this geometry as constants;
+    MXD_MSDA_BWD_FIXED=0 sends them through the general one.  Both against the oracle, and the gradients of locations and
+    weights (which do not depend on the order of any sum) bit for bit against each other; the query count leaves the last
+    workgroup partly filled."""
+    levels = ((37, 52), (19, 26), (10, 13), (5, 7))[:nl]
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh, hd = 2, 1237, 8, 32
+    g = torch.Generator().manual_seed(7 * nl + npts)
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g).to(dtype), shapes, lsi,
+                               (torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.2 - 0.1).to(dtype),
+                               torch.rand(bs, nq, nh, nl, npts, generator=g).to(dtype),
+                               torch.randn(bs, nq, nh * hd, generator=g).to(dtype))
+    plan = _lib.make_plan(1, {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype], bs, nk, nh, hd, nl, nl, nq, npts)
+    assert plan.lanes_per_row == 8 and plan.units_per_wave == 8 and plan.iters == 1
+    tol = (FWD_FP32, BWD_FP32) if dtype == torch.float32 else (half_tol(dtype),) * 2
+    got = {}
+    for fixed in ("1", "0"):
+        set_tuning(monkeypatch, MXD_MSDA_BWD_FIXED=fixed)
+        _check_all(inp, gpu_device, *tol)
+        got[fixed] = run_gpu(inp, gpu_device)
+    assert np.array_equal(got["1"][2], got["0"][2]) and np.array_equal(got["1"][3], got["0"][3])
+
+
 @pytest.mark.parametrize("lds", ["0", "2048", "32768", "49152", "65536"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
