@@ -466,7 +466,7 @@ def _bench_heuristics(args):
                     {"MXD_MSDA_FWD_CU": 0, "MXD_MSDA_FWD_LDS": 40960}, {"MXD_MSDA_FWD_CU_FLIP": 0}, {"MXD_MSDA_FWD_CU_FLIP": 1}]
     bwd_variants = [{}, {"MXD_MSDA_BWD_UNIT_SPLIT": 0}, {"MXD_MSDA_BWD_UNIT_SPLIT": 2}, {"MXD_MSDA_TILE_PX_LOG2": 9}, {"MXD_MSDA_TILE_PX_LOG2": 8},
                     {"MXD_MSDA_TILE_PX_LOG2": 7}, {"MXD_MSDA_BWD_REC_LDS": 0}, {"MXD_MSDA_BWD_REC_LDS": 1},
-                    {"MXD_MSDA_BWD_LANE_BYTES": 16}, {"MXD_MSDA_BWD_LANE_BYTES": 8}]
+                    {"MXD_MSDA_BWD_LANE_BYTES": 16}, {"MXD_MSDA_BWD_LANE_BYTES": 8}, {"MXD_MSDA_BWD_FIXED": 0}]
     saved = {k: v for k, v in os.environ.items() if k.startswith("MXD_MSDA_")}
 
     def set_env(env):
@@ -524,7 +524,7 @@ def _bench_heuristics(args):
                     if env and rep == 0:
                         same[label(env)] = _lib.make_plan(what == "backward", code, *dims).as_dict() == plan0 and \
                             not any(k in env for k in ("MXD_MSDA_FWD_CU_FLIP", "MXD_MSDA_TILE_PX_LOG2", "MXD_MSDA_BWD_REC_LDS",
-                                                       "MXD_MSDA_BWD_UNIT_SPLIT"))
+                                                       "MXD_MSDA_BWD_UNIT_SPLIT", "MXD_MSDA_BWD_FIXED"))
                     if same.get(label(env)):
                         continue
                     t = _event_ms(fn, iters, iters) * 1e3
