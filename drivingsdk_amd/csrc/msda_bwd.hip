@@ -454,33 +454,78 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
             // uniform branches keep the row loads of the next samples from being issued early)
             auto gather_dots = [&](auto lg) {
                 constexpr int LG = decltype(lg)::value;
-                for (int sl = 0; sl < ns; ++sl) {
+                typedef typename RowIO<T, VEC>::raw_t raw_t;
+                // the corner rows of staged sample sl (channels of row pass p)
+                auto request = [&](int sl, int p, raw_t (&raw)[NC]) {
                     const u32x4 off = *reinterpret_cast<const u32x4*>(mine[sl].off);
-                    float d[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int p = 0; p < NPASS; ++p) {
-                        typename RowIO<T, VEC>::raw_t raw[NC];
+                    for (int k = 0; k < NC; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
+                };
+                auto accumulate = [&](int p, const raw_t (&raw)[NC], float (&d)[4]) {
 #pragma unroll
-                        for (int k = 0; k < NC; ++k) raw[k] = RowIO<T, VEC>::load_raw(vres, off[k] + choff[p]);
+                    for (int k = 0; k < NC; ++k) {
+                        if constexpr (kDot2) {
+                            uint32_t words[kPairs];
+                            __builtin_memcpy(words, &raw[k], sizeof(words));
 #pragma unroll
-                        for (int k = 0; k < NC; ++k) {
-                            if constexpr (kDot2) {
-                                uint32_t words[kPairs];
-                                __builtin_memcpy(words, &raw[k], sizeof(words));
+                            for (int e = 0; e < kPairs; ++e) d[k] = dot2_acc<T>(words[e], gpk[p][e], d[k]);
+                        } else {
+                            float v[VEC];
+                            RowIO<T, VEC>::unpack(raw[k], v);
 #pragma unroll
-                                for (int e = 0; e < kPairs; ++e) d[k] = dot2_acc<T>(words[e], gpk[p][e], d[k]);
-                            } else {
-                                float v[VEC];
-                                RowIO<T, VEC>::unpack(raw[k], v);
-#pragma unroll
-                                for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
-                            }
+                            for (int e = 0; e < VEC; ++e) d[k] = __builtin_fmaf(v[e], gv[p][e], d[k]);
                         }
                     }
+                };
+                auto finish = [&](int sl, const float (&d)[4]) {
                     f32x4 dsum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int k = 0; k < NC; ++k) dsum[k] = group_sum<LG>(d[k]);
                     if (c == 0) dots[g * kChunk + sl] = dsum;
+                };
+                // (where it measured faster: the fixed geometry, and geometric kernel attention -- step 0.807 -> 0.786 ms;
+                //  the fused form, 0.440 -> 0.459 ms for forward + backward, and the grid sampler, 0.192 -> 0.200 ms, lose
+                //  more to the registers than they gain)
+                constexpr bool kAhead = (FIXED != 0 || SRC == kSrcGka) && NPASS <= 2;
+                if constexpr (kAhead) {
+                    // the rows of the next sample (of the row's second half, with two passes) are requested before the
+                    // rows at hand are used: a wavefront otherwise goes through the samples of its chunk one trip to
+                    // memory after the other, and spends 71 % of its life in this loop (encoder backward 268.4 ->
+                    // 260.9 us, float16 277.5 -> 270.3, BEVFormer shape 998 -> 994; with three sets of rows in flight
+                    // the encoder shape loses 1.5 us to the registers they take)
+                    raw_t ra[NC], rb[NC];
+                    constexpr int PB = NPASS - 1;  // row pass of the second set
+                    float d[4] = {0.f, 0.f, 0.f, 0.f};
+                    auto consume = [&](int t, auto pass, const raw_t (&raw)[NC]) {
+                        constexpr int P = decltype(pass)::value;
+                        accumulate(P, raw, d);
+                        if (P == NPASS - 1) {
+                            finish(t / NPASS, d);
+                            d[0] = d[1] = d[2] = d[3] = 0.f;
+                        }
+                    };
+                    const int nt = ns * NPASS;  // (even with two passes)
+                    request(0, 0, ra);
+                    for (int t = 0; t < nt; t += 2) {
+                        const bool two = t + 1 < nt;
+                        if (two) request((t + 1) / NPASS, PB, rb);
+                        consume(t, std::integral_constant<int, 0>{}, ra);
+                        if (two) {
+                            if (t + 2 < nt) request((t + 2) / NPASS, 0, ra);
+                            consume(t + 1, std::integral_constant<int, PB>{}, rb);
+                        }
+                    }
+                } else {
+                    for (int sl = 0; sl < ns; ++sl) {
+                        float d[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int p = 0; p < NPASS; ++p) {
+                            raw_t raw[NC];
+                            request(sl, p, raw);
+                            accumulate(p, raw, d);
+                        }
+                        finish(sl, d);
+                    }
                 }
             };
             switch (lpr_log2) {
