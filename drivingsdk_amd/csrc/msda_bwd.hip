@@ -377,7 +377,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
                     if (lane >= d) inc += o;
                 }
                 if (i < a.tbl_stride) cursor[i] = carry + inc - v;
-                carry += __shfl(inc, kWave - 1, kWave);
+                carry += __builtin_amdgcn_readlane(inc, kWave - 1);
             }
         }
         __syncthreads();
