@@ -5,7 +5,7 @@ import subprocess
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def build(force=True, jobs=4, verbose=False):
+def build(force=True, jobs=8, verbose=False):
     """Compile the HIP sources under ``csrc/`` into ``lib/libmxd_msda.so``.  Returns its path."""
     cmd = ["make", "-C", os.path.join(_HERE, "csrc"), f"-j{jobs}"]
     if force:

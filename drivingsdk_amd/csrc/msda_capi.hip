@@ -1,5 +1,5 @@
 // C ABI entry points (include/mxd_msda.h): argument checks, launch geometry, enqueue.
-// Host code only; the kernels live in msda_fwd.hip, msda_bwd.hip and msda_bwd_tiles.hip.  Multi-scale
+// Host code only; the kernels live in msda_fwd.hip, msda_fwd_cu.hip, msda_bwd_kernel.h (with msda_bwd*.hip) and msda_bwd_tiles.hip.  Multi-scale
 // deformable attention, its fused form, deformable aggregation and geometric kernel attention are the same
 // three kernels with different sample sources (msda_device.h: sample_ref, source_geometry).
 #include <hip/hip_runtime.h>
@@ -390,7 +390,7 @@ size_t bwd_workspace_bytes(int dtype, const Dims& d)
     return a > b ? a : b;
 }
 
-// LDS for the slab of a workgroup of the first backward kernel that makes several passes (msda_bwd.hip): 12 bytes per
+// LDS for the slab of a workgroup of the first backward kernel that makes several passes (msda_bwd_kernel.h): 12 bytes per
 // record behind the counters, when the slab is small enough to leave four workgroups to a CU and the kernel stays
 // inside the default limit of dynamic LDS.  A workgroup that makes one pass of one chunk (the plain operator and the
 // fused form) collects its records in its staging strips instead.  Adds the bytes to the plan.
