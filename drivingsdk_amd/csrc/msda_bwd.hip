@@ -34,10 +34,16 @@ __global__ __launch_bounds__(256) void msda_round_kernel(const float* src, T* ds
 template <typename T>
 __global__ __launch_bounds__(256) void msda_round_rows_kernel(const KArgs a)
 {
+    // the levels through LDS, one per thread: evaluated straight from memory the two tests below are a chain of scalar
+    // loads, one level after the other, in front of a workgroup that moves a few kilobytes
+    __shared__ i32x4 lv[kMaxLevels];
+    if ((int)threadIdx.x < a.nl) lv[threadIdx.x] = load_level(a, (int)threadIdx.x);
+    __syncthreads();
+    auto level = [&](int l) { return lv[l]; };
     const int32_t tiles = a.tbl_stride - 1;
     const uint32_t row4 = (uint32_t)(a.nh * a.hd) / 4;
     typedef T t4 __attribute__((ext_vector_type(4)));
-    if (!levels_tile_the_keys(a)) {
+    if (!levels_tile_the_keys_of(a, level)) {
         // every row went through the fp32 image: the workgroups round it between them
         const uint64_t n4 = (uint64_t)a.bs * a.nk * row4, per = (n4 + gridDim.x - 1) / gridDim.x;
         const uint64_t lo = (uint64_t)blockIdx.x * per, hi = lo + per < n4 ? lo + per : n4;
@@ -51,7 +57,7 @@ __global__ __launch_bounds__(256) void msda_round_rows_kernel(const KArgs a)
     }
     const int32_t b = (int32_t)(blockIdx.x / (uint32_t)(tiles * kRowParts)), r = (int32_t)(blockIdx.x % (uint32_t)(tiles * kRowParts));
     int32_t r0, r1;
-    if (b >= a.bs || !atomic_rows_of_part(a, r / kRowParts, r % kRowParts, &r0, &r1)) return;
+    if (b >= a.bs || !atomic_rows_of_part_of(a, level, r / kRowParts, r % kRowParts, &r0, &r1)) return;
     const f32x4* src = reinterpret_cast<const f32x4*>(a.grad_value) + ((size_t)b * a.nk + r0) * row4;
     t4* dst = reinterpret_cast<t4*>(a.grad_value_t) + ((size_t)b * a.nk + r0) * row4;
     const uint32_t n4 = (uint32_t)(r1 - r0) * row4;

@@ -148,12 +148,14 @@ __device__ inline bool tile_stored_directly(int32_t chunks, int32_t npx, int32_t
 // them) and lets the rows that nobody adds to go without zeros.  level_start_index is the caller's: for any other
 // layout (keys that no level covers, levels out of order or overlapping) every row is zero-filled and every tile adds
 // its sums with atomics.
-__device__ inline bool levels_tile_the_keys(const KArgs& a)
+// (level(l): {H, W, first key} of level l, from wherever the caller holds it)
+template <typename GetLevel>
+__device__ inline bool levels_tile_the_keys_of(const KArgs& a, GetLevel level)
 {
     int64_t next = 0;
     int32_t tiles = 0;
     for (int l = 0; l < a.nl; ++l) {
-        const i32x4 L = load_level(a, l);
+        const i32x4 L = level(l);
         if (L.x <= 0 || L.y <= 0 || (int64_t)L.z != next) return false;
         const int64_t px = (int64_t)L.x * L.y;
         next += px;
@@ -162,15 +164,20 @@ __device__ inline bool levels_tile_the_keys(const KArgs& a)
     }
     return next == a.nk && tiles <= a.tbl_stride - 1;
 }
+__device__ inline bool levels_tile_the_keys(const KArgs& a)
+{
+    return levels_tile_the_keys_of(a, [&](int l) { return load_level(a, l); });
+}
 
 // Rows (pixels of a batch element) [*r0, *r1) of piece `part` (< kRowParts) of tile `tile` of a batch element that
 // receive atomic additions in the tile pass; false when there is no such tile.  Tiles are numbered level by level as
 // in the first kernel and the tile pass.
-__device__ inline bool atomic_rows_of_part(const KArgs& a, int32_t tile, int32_t part, int32_t* r0, int32_t* r1)
+template <typename GetLevel>
+__device__ inline bool atomic_rows_of_part_of(const KArgs& a, GetLevel level, int32_t tile, int32_t part, int32_t* r0, int32_t* r1)
 {
     int32_t first = 0;
     for (int l = 0; l < a.nl; ++l) {
-        const i32x4 L = load_level(a, l);
+        const i32x4 L = level(l);
         int32_t P;
         const int32_t nt = level_tile_count(L.x, L.y, L.z, a.nk, a.tile_px_log2, &P);
         if (first + nt > a.tbl_stride - 1) continue;  // (a level that does not fit the run table has no tiles)
@@ -192,6 +199,10 @@ __device__ inline bool atomic_rows_of_part(const KArgs& a, int32_t tile, int32_t
         first += nt;
     }
     return false;
+}
+__device__ inline bool atomic_rows_of_part(const KArgs& a, int32_t tile, int32_t part, int32_t* r0, int32_t* r1)
+{
+    return atomic_rows_of_part_of(a, [&](int l) { return load_level(a, l); }, tile, part, r0, r1);
 }
 
 // Where a kernel takes the location and the weight of sample s of unit (b, q, h) from.
