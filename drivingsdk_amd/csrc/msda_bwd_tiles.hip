@@ -212,7 +212,7 @@ __global__ __launch_bounds__(kTileThreads, 4) void msda_gradv_tiles_kernel(const
     // (a wavefront transposes the sums of half of its lane groups at a time: 4 groups x 32 sums x 8 lanes = 4 KiB)
     constexpr int kSlotPxAt = 4 * PPG * CH / 4;         // first entry behind wavefront 0's transposition scratch
     static_assert(kSlotPxAt + kTileThreads * 2 / 16 <= kCarryAt, "slot map must fit wavefront 0's entry storage");
-    __shared__ uint32_t heads[kTileThreads];            // list head per pixel slot (entry index)
+    __shared__ uint32_t heads[kTileThreads];            // list head per pixel slot (byte offset of the entry in `ent`)
     // entry: {byte offset of the grad_out row, weight for the list's pixel, weight for the
     // next pixel, next entry of the same list}
     __shared__ u32x4 ent[NW * kTileEntCap];
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(kTileThreads, 4) void msda_gradv_tiles_kernel(const
     if (threadIdx.x < kTileThreads / 2) slot_info[threadIdx.x] = 0;
     // an empty list points at the dummy entry of the wavefront that owns the pixel slot (slot s belongs to lane group
     // s / PPG, i.e. to wavefront s / (8 PPG); slots past the tile size are never used)
-    heads[threadIdx.x] = (threadIdx.x / (kLpp * PPG)) % NW * kTileEntCap + kDummyOfWave;
+    heads[threadIdx.x] = ((threadIdx.x / (kLpp * PPG)) % NW * kTileEntCap + kDummyOfWave) * 16u;
     __syncthreads();
     if (threadIdx.x == 0) {
         item_ok = decode_tile_item(a, t, lv_info, wk.q_begin, &item_s, lv_first, lv_nt) ? 1 : 0;
@@ -313,8 +313,10 @@ __global__ __launch_bounds__(kTileThreads, 4) void msda_gradv_tiles_kernel(const
     const uint32_t ghead_off = (uint32_t)wk.h * hd * (uint32_t)sizeof(T);
     // the dummy entry ends every list of this wavefront's pixels: weight 0, a row offset the
     // buffer range check answers with zeros (at no cost in the memory pipeline), next = itself
-    const uint32_t dummy = seg + kDummyOfWave;
-    if (lane == 0) ent[dummy] = u32x4{kInvalidCorner, 0u, 0u, dummy};
+    // (lists are linked by byte offsets into `ent`: the walk then needs no shift per entry)
+    const uint32_t dummy = (seg + kDummyOfWave) * 16u;
+    auto ent_at = [&](uint32_t off) -> u32x4& { return *reinterpret_cast<u32x4*>(reinterpret_cast<unsigned char*>(ent) + off); };
+    if (lane == 0) ent_at(dummy) = u32x4{kInvalidCorner, 0u, 0u, dummy};
 
     // lane j of group g = tid / 8 keeps channels 32k + 4j .. 32k + 4j + 3 (k < NB) of the pixels g*PPG .. g*PPG + PPG - 1
     const int grp = tid / kLpp, j = tid % kLpp;
@@ -458,7 +460,7 @@ __global__ __launch_bounds__(kTileThreads, 4) void msda_gradv_tiles_kernel(const
                             const uint32_t pos = seg + count +
                                                  __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
                                                                            __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
-                            const uint32_t next = atomicExch(&heads[lst[k]], pos);
+                            const uint32_t next = atomicExch(&heads[lst[k]], pos * 16u);
                             ent[pos] = u32x4{q * row_bytes, __builtin_bit_cast(uint32_t, w0[k]),
                                              __builtin_bit_cast(uint32_t, w1[k]), next};
                             if (count_slots) atomicAdd(&slot_info[lst[k] >> 1], (lst[k] & 1) ? 0x10000u : 1u);
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(kTileThreads, 4) void msda_gradv_tiles_kernel(const
             // kWalk lists are walked together, one entry of each per trip, and two trips are in flight.
             {
                 auto fetch = [&](uint32_t& e, float (&g)[CHL], float& wa, float& wb) {
-                    const u32x4 en = ent[e];
+                    const u32x4 en = ent_at(e);
                     // (a bit cast applied directly to a vector element picks up element 0: copy first)
                     const uint32_t ya = en.y, za = en.z;
                     wa = __builtin_bit_cast(float, ya);
@@ -711,7 +713,7 @@ __global__ __launch_bounds__(kTileThreads, 4) void msda_gradv_tiles_kernel(const
             // overwritten by the transposition)
             __syncthreads();
             if (threadIdx.x == 0) done_count = 0;
-            if (lane == 0) ent[dummy] = u32x4{kInvalidCorner, 0u, 0u, dummy};
+            if (lane == 0) ent_at(dummy) = u32x4{kInvalidCorner, 0u, 0u, dummy};
             __syncthreads();
         }
     }
