@@ -45,10 +45,16 @@ namespace mxd {
 // wavefront), one iteration of one chunk, the plain operator's tile form, with a unit per query (1: up to 16 samples per
 // query) or two (2: up to 32): the paths for anything else and the scalar registers that steer them fall away (57
 // vector registers instead of 96 and no spilled scalar ones; encoder shape 281.7 -> 276.3 us, float16 294.0 -> 286.7).
+// FIXED == 3: rows of 256 bytes read by 16 lanes (4 units per wavefront), a unit per query, any number of iterations
+// and chunks (heads of 128 channels in the 16-bit types: backward 380.2 -> 366.1 us in float16, 382.9 -> 369.7 in bfloat16).
 template <typename T, int VEC, int NPASS, bool SCATTER, int SRC, bool RECBUF = false, int FIXED = 0>
 __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
-    static_assert(!FIXED || (!SCATTER && !RECBUF && SRC == kSrcPlain), "the fixed geometry is built for the plain operator's tile form");
+    static_assert(!FIXED || (!SCATTER && SRC == kSrcPlain), "the fixed geometry is built for the plain operator's tile form");
+    // 1, 2: 8 lanes per row, one pass of one chunk, one / two units per query; 3: 16 lanes per row (4 units per wavefront), a
+    // unit per query, any number of iterations and chunks (rows of 256 bytes: heads of 128 channels in the 16-bit types)
+    constexpr bool kOnePass = FIXED == 1 || FIXED == 2;
+    static_assert(!(kOnePass && RECBUF), "a workgroup that makes one pass collects its records in its staging strips");
     static_assert(!RECBUF || (!SCATTER && (SRC == kSrcPlain || SRC == kSrcFused)), "the record buffer is built for the tile form of the operator and its fused form");
     constexpr int GSHIFT = sizeof(T) == 4 ? 0 : 1;  // value byte offset -> fp32 image byte offset
     constexpr bool FUSED = SRC == kSrcFused;
@@ -98,13 +104,13 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
 
-    const int LPR = FIXED ? 8 : a.plan.lanes_per_row;
-    const int lpr_log2 = FIXED ? 3 : __builtin_ctz(LPR);
-    const int U = FIXED ? 8 : a.plan.units_per_wave;
-    const int iters = FIXED ? 1 : a.plan.iters;
+    const int LPR = FIXED == 3 ? 16 : FIXED ? 8 : a.plan.lanes_per_row;
+    const int lpr_log2 = FIXED == 3 ? 4 : FIXED ? 3 : __builtin_ctz(LPR);
+    const int U = FIXED == 3 ? 4 : FIXED ? 8 : a.plan.units_per_wave;
+    const int iters = kOnePass ? 1 : a.plan.iters;
     // 2^sp neighbouring units share a query, each taking kChunk of its samples: a pass of a wavefront covers `span`
     // samples of U >> sp queries (sp = 0: a unit is a query and goes through its samples kChunk at a time)
-    const int sp = FIXED ? FIXED - 1 : a.unit_split_log2, sp_mask = (1 << sp) - 1, span = kChunk << sp;
+    const int sp = FIXED == 3 ? 0 : FIXED ? FIXED - 1 : a.unit_split_log2, sp_mask = (1 << sp) - 1, span = kChunk << sp;
     const int g = lane >> lpr_log2;
     const int c = lane & (LPR - 1);
     // lanes per row in the scatter phase: the power of two covering head_dim, within [LPR, 64]
@@ -337,7 +343,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
         // the workgroup goes through every trip (the lane exchanges need their partners).
         const int S4 = (a.S + 3) & ~3;
         const int n = (wk.q_end - wk.q_begin) * S4;
-        const bool all_early = FIXED || (early_units >= wk.q_end - wk.q_begin && a.S <= span);  // nothing left to count
+        const bool all_early = kOnePass || (early_units >= wk.q_end - wk.q_begin && a.S <= span);  // nothing left to count
         for (int base = 0; base < n && !all_early; base += blockDim.x) {
             const int i = base + (int)threadIdx.x;
             const int qr = i / S4, s = i - qr * S4;
@@ -404,8 +410,8 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
     // wavefront has gathered, the staged entries are free, and a unit's 32 records (two per sample) fit the 16 entries
     // before its pad entry (which the fused form still needs).  Record `pos` of the slab lives at record pos % 32 of
     // unit pos / 32 of the workgroup.
-    const bool rec_in_lds = FIXED || ((SRC == kSrcPlain || SRC == kSrcFused) && !SCATTER && iters == 1 && a.S <= span);
-    const int u_log2 = FIXED ? 3 : __builtin_ctz(U);
+    const bool rec_in_lds = kOnePass || ((SRC == kSrcPlain || SRC == kSrcFused) && !SCATTER && iters == 1 && a.S <= span);
+    const int u_log2 = FIXED == 3 ? 2 : FIXED ? 3 : __builtin_ctz(U);
     auto rec_lds = [&](int pos) {
         const int unit = pos >> 5;  // of the workgroup: wavefront unit >> u_log2, its unit & (U - 1)
         return reinterpret_cast<u32x4*>(smem + kMaxLevels * sizeof(i32x4) +
@@ -448,7 +454,7 @@ __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 
         if (!(kEarly && FUSED && it == 0)) unit_prologue(q0);  // (the fused form's first iteration: done before the count)
 
-        for (int c0 = 0; c0 < (FIXED ? 1 : a.S); c0 += span) {
+        for (int c0 = 0; c0 < (kOnePass ? 1 : a.S); c0 += span) {
             // ---- geometry (the first chunk of the first iteration was staged while records were counted) ----
             if (!(kEarly && it == 0 && c0 == 0)) geometry(q0, c0, std::false_type{});
             wave_lds_sync();
@@ -784,6 +790,9 @@ template <typename T, int VEC, int NPASS>
 inline hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
 {
     const dim3 grid(a.plan.grid), block(a.plan.block);
+    // (the 16-lane fixed geometry is built for lanes of 16 bytes and one row pass: rows of 256 bytes; with two passes --
+    //  heads of 128 float32 channels -- it changes nothing, 544 us)
+    constexpr bool kWide = sizeof(T) * VEC == 16 && NPASS == 1;
     if (a.grid) {
         if (scatter)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcGrid>), grid, block, a.plan.lds_bytes, stream, a);
@@ -809,6 +818,10 @@ inline hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
     } else {
         if (scatter)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcPlain>), grid, block, a.plan.lds_bytes, stream, a);
+        else if (a.bwd_fixed == 3 && kWide && a.rec_lds_bytes != 0)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, kWide ? NPASS : 1, false, kSrcPlain, true, 3>), grid, block, a.plan.lds_bytes, stream, a);
+        else if (a.bwd_fixed == 3 && kWide)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, kWide ? NPASS : 1, false, kSrcPlain, false, 3>), grid, block, a.plan.lds_bytes, stream, a);
         else if (a.rec_lds_bytes != 0)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcPlain, true>), grid, block, a.plan.lds_bytes, stream, a);
         else if (a.bwd_fixed == 1 && NPASS == 1)

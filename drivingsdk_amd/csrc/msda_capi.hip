@@ -1031,6 +1031,9 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
                    a.plan.npass == 1 && a.plan.iters == 1 && a.unit_split_log2 <= 1 &&
                    d.nl * d.np <= ((int64_t)mxd::kChunk << a.unit_split_log2) && a.rec_lds_bytes == 0)
                       ? 1 + a.unit_split_log2 : 0;
+    if (tuning().bwd_fixed != 0 && !fused && !gka && !grid && L.tiles && a.plan.lanes_per_row == 16 && a.plan.units_per_wave == 4 &&
+        a.plan.npass == 1 && a.plan.vec * (int)elem_size(dtype) == 16 && a.unit_split_log2 == 0)
+        a.bwd_fixed = 3;
     a.meta_i64 = meta64;
     a.value = value;
     a.shapes = spatial_shapes;

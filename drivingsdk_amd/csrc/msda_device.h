@@ -72,8 +72,8 @@ struct KArgs {
     int32_t rec_lds_bytes; // first backward kernel: LDS behind its counters (16-byte aligned) in which a workgroup that makes
                            // several passes collects its slab before it writes it; 0 = none (records stored one by one)
     int32_t bwd_fixed;     // first backward kernel, plain operator's tile form: 1, 2 = the launch has the common geometry (rows read
-                           // by 8 lanes, one iteration of one chunk, this many units per query) and takes the instantiation built
-                           // for it
+                           // by 8 lanes, one iteration of one chunk, this many units per query), 3 = rows of 256 bytes read by 16
+                           // lanes of 16 bytes, a unit per query: it takes the instantiation built for that geometry
     int32_t tile_target;   // pair records per work item of the tile pass aimed at when a hot tile is split by query range
     int32_t tile_max_chunks;  // most query chunks a tile is split into
     int32_t sparse;        // 1: only the rows of the image that receive atomic additions are zero-filled (and, for 16-bit

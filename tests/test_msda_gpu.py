@@ -562,6 +562,37 @@ def test_first_backward_kernel_with_its_geometry_as_constants(gpu_device, monkey
     assert np.array_equal(got["1"][2], got["0"][2]) and np.array_equal(got["1"][3], got["0"][3])
 
 
+@pytest.mark.parametrize("rec_lds", ["0", "1"], ids=["records-stored-singly", "slab-in-lds"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("nl,npts", [(4, 4), (3, 5), (1, 1), (4, 8), (2, 13)])
+def test_first_backward_kernel_with_rows_of_256_bytes_as_constants(gpu_device, monkeypatch, nl, npts, dtype, rec_lds):
+    """Rows of 256 bytes (64 float32 channels, 128 channels of a 16-bit type) are read by 16 lanes of 16 bytes, four units
+    per wavefront: such launches take an instantiation of the first backward kernel with that geometry as constants,
+    whatever their number of iterations and chunks (here one to two chunks per query), with the records stored one by one
+    or collected in LDS.  Against the oracle, and the gradients of locations and weights bit for bit against the general
+    instantiation (MXD_MSDA_BWD_FIXED=0)."""
+    levels = ((37, 52), (19, 26), (10, 13), (5, 7))[:nl]
+    shapes, lsi = workloads.level_tensors(levels)
+    nk = int(shapes.prod(1).sum())
+    bs, nq, nh = 2, 1237, 3
+    hd = 64 if dtype == torch.float32 else 128
+    g = torch.Generator().manual_seed(11 * nl + npts)
+    inp = workloads.MsdaInputs(torch.randn(bs, nk, nh, hd, generator=g).to(dtype), shapes, lsi,
+                               (torch.rand(bs, nq, nh, nl, npts, 2, generator=g) * 1.2 - 0.1).to(dtype),
+                               torch.rand(bs, nq, nh, nl, npts, generator=g).to(dtype),
+                               torch.randn(bs, nq, nh * hd, generator=g).to(dtype))
+    set_tuning(monkeypatch, MXD_MSDA_BWD_REC_LDS=rec_lds)
+    plan = _lib.make_plan(1, {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype], bs, nk, nh, hd, nl, nl, nq, npts)
+    assert plan.lanes_per_row == 16 and plan.units_per_wave == 4 and plan.npass == 1
+    tol = (FWD_FP32, BWD_FP32) if dtype == torch.float32 else (half_tol(dtype),) * 2
+    got = {}
+    for fixed in ("1", "0"):
+        set_tuning(monkeypatch, MXD_MSDA_BWD_REC_LDS=rec_lds, MXD_MSDA_BWD_FIXED=fixed)
+        _check_all(inp, gpu_device, *tol)
+        got[fixed] = run_gpu(inp, gpu_device)
+    assert np.array_equal(got["1"][2], got["0"][2]) and np.array_equal(got["1"][3], got["0"][3])
+
+
 @pytest.mark.parametrize("lds", ["0", "2048", "32768", "49152", "65536"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
 def test_forward_level_cache_sizes(gpu_device, monkeypatch, lds, dtype):
