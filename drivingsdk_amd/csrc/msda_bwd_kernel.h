@@ -50,7 +50,8 @@ namespace mxd {
 template <typename T, int VEC, int NPASS, bool SCATTER, int SRC, bool RECBUF = false, int FIXED = 0>
 __global__ __launch_bounds__(256) void msda_bwd_kernel(const KArgs a)
 {
-    static_assert(!FIXED || (!SCATTER && SRC == kSrcPlain), "the fixed geometry is built for the plain operator's tile form");
+    static_assert(!FIXED || (!SCATTER && (SRC == kSrcPlain || (SRC == kSrcFused && FIXED == 1))),
+                  "the fixed geometry is built for the tile form of the plain operator (and, one unit per query in one pass, of its fused form)");
     // 1, 2: 8 lanes per row, one pass of one chunk, one / two units per query; 3: 16 lanes per row (4 units per wavefront), a
     // unit per query, any number of iterations and chunks (rows of 256 bytes: heads of 128 channels in the 16-bit types)
     constexpr bool kOnePass = FIXED == 1 || FIXED == 2;
@@ -813,6 +814,8 @@ inline hipError_t launch_one(const KArgs& a, bool scatter, hipStream_t stream)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, true, kSrcFused>), grid, block, a.plan.lds_bytes, stream, a);
         else if (a.rec_lds_bytes != 0)
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcFused, true>), grid, block, a.plan.lds_bytes, stream, a);
+        else if (a.bwd_fixed == 1 && NPASS == 1)
+            hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, 1, false, kSrcFused, false, 1>), grid, block, a.plan.lds_bytes, stream, a);
         else
             hipLaunchKernelGGL((msda_bwd_kernel<T, VEC, NPASS, false, kSrcFused>), grid, block, a.plan.lds_bytes, stream, a);
     } else {

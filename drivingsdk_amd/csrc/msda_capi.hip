@@ -1027,8 +1027,8 @@ static int backward_common(int kind, const void* value, const int32_t* spatial_s
     a.tile_px_log2 = L.tile_px_log2;
     a.unit_split_log2 = unit_split_log2(a.plan);
     a.rec_lds_bytes = plan_record_buffer(&a.plan, L, d, dtype, !gka && !grid, a.unit_split_log2);
-    a.bwd_fixed = (tuning().bwd_fixed != 0 && !fused && !gka && !grid && L.tiles && a.plan.lanes_per_row == 8 && a.plan.units_per_wave == 8 &&
-                   a.plan.npass == 1 && a.plan.iters == 1 && a.unit_split_log2 <= 1 &&
+    a.bwd_fixed = (tuning().bwd_fixed != 0 && (!fused || a.unit_split_log2 == 0) && !gka && !grid && L.tiles && a.plan.lanes_per_row == 8 &&
+                   a.plan.units_per_wave == 8 && a.plan.npass == 1 && a.plan.iters == 1 && a.unit_split_log2 <= 1 &&
                    d.nl * d.np <= ((int64_t)mxd::kChunk << a.unit_split_log2) && a.rec_lds_bytes == 0)
                       ? 1 + a.unit_split_log2 : 0;
     if (tuning().bwd_fixed != 0 && !fused && !gka && !grid && L.tiles && a.plan.lanes_per_row == 16 && a.plan.units_per_wave == 4 &&

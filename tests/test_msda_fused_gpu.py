@@ -74,9 +74,13 @@ def _run(value, shapes, lsi, ref, off, logits, grad_out, device):
     return [t.detach().double().cpu().numpy() for t in (out, v.grad, r.grad, o.grad, z.grad)]
 
 
+@pytest.mark.parametrize("fixed", ["1", "0"], ids=["geometry-as-constants", "general-first-kernel"])
 @pytest.mark.parametrize("name,ref_dim,scale", [("tiny", 2, 1.0), ("tiny", 4, 1.0), ("detr_encoder", 2, 0.25),
                                                 ("bevformer_sca", 2, 0.1)])
-def test_fused_forward_and_gradients_fp32(gpu_device, name, ref_dim, scale):
+def test_fused_forward_and_gradients_fp32(gpu_device, monkeypatch, name, ref_dim, scale, fixed):
+    """(The backward's first kernel has an instantiation with the launch geometry of up to 16 samples per query as
+    constants, which the tiny and encoder shapes take by default; MXD_MSDA_BWD_FIXED=0 sends them through the general one.)"""
+    set_tuning(monkeypatch, MXD_MSDA_BWD_FIXED=fixed)
     inp = make_fused_inputs(name, ref_dim, scale)
     value, shapes, lsi, ref, off, logits, grad_out = inp
     want = orc.fused_fwd_bwd(value, shapes, ref, off, logits, grad_out, loc_dtype=torch.float32)
