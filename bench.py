@@ -172,17 +172,31 @@ def _module_forward_times(d, iters, warmup):
     return res
 
 
+def kernel_sources_digest():
+    """SHA-256 over the HIP sources of the library (csrc/*.hip, *.h and the public header): which kernels a committed
+    counter measurement was taken with."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "drivingsdk_amd", "csrc")
+    files = sorted(f for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
+    for path in [os.path.join(csrc, f) for f in files] + [os.path.join(ROOT, "include", "mxd_msda.h")]:
+        with open(path, "rb") as f:
+            h.update(os.path.basename(path).encode() + b"\0" + f.read() + b"\0")
+    return h.hexdigest()
+
+
 def _committed_traffic(workload, dtype):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
-    kernel of known size) and committed under profiles/; None when no measurement covers this run."""
+    kernel of known size) and committed under profiles/; (None, None) when no measurement covers this run.
+    Second value: whether the measurement was taken with the kernel sources of this tree."""
     path = os.path.join(ROOT, "profiles", "traffic_detr_encoder_fp32.json")
     if not os.path.exists(path):
-        return None
+        return None, None
     with open(path) as f:
         data = json.load(f)
     if data.get("workload") != workload or data.get("dtype") != dtype:
-        return None
-    return data["kernels"]
+        return None, None
+    return data["kernels"], data.get("kernel_sources_sha256") == kernel_sources_digest()
 
 
 def _physical_cores():
@@ -629,7 +643,7 @@ def main():
     bytes_fwd = workloads.algorithmic_bytes(inp, backward=False)
     bytes_bwd = workloads.algorithmic_bytes(inp, backward=True)
 
-    traffic = _committed_traffic(args.workload, args.dtype)
+    traffic, traffic_current = _committed_traffic(args.workload, args.dtype)
     copy_gbps = _copy_bandwidth_gbps()
 
     def roof(nbytes, ms, kernels):
@@ -637,9 +651,14 @@ def main():
         hbm = None
         if traffic is not None and all(k in traffic for k in kernels):
             hbm = sum(traffic[k]["hbm_bytes"] for k in kernels)
-        return {"bound": "hbm", "kernel": " + ".join(kernels), "achieved": achieved, "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": hbm, "algorithmic_bytes": nbytes,
-                "kernel_ms": ms, "measured_copy_GBps": copy_gbps, "frac_of_measured_copy": achieved / copy_gbps}
+        r = {"bound": "hbm", "kernel": " + ".join(kernels), "achieved": achieved, "peak": HBM_PEAK_GBPS,
+             "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": hbm, "algorithmic_bytes": nbytes,
+             "kernel_ms": ms, "measured_copy_GBps": copy_gbps, "frac_of_measured_copy": achieved / copy_gbps}
+        if hbm is not None:
+            # (a committed rocprofv3 --pmc measurement, not a figure of this run: taken with these kernel sources or not)
+            r["traffic_from"] = "profiles/traffic_detr_encoder_fp32.json"
+            r["traffic_measured_with_these_kernel_sources"] = bool(traffic_current)
+        return r
 
     roof_fwd = roof(bytes_fwd, k["forward_ms"], [k["forward_kernel"]])
     # the backward pass: per-sample dots (grad_attn, grad_loc, records; its workgroups also zero-fill the image),

@@ -39,6 +39,8 @@ def test_default_workload_line(gpu_device):
         assert abs(f["achieved"] - f["algorithmic_bytes"] / (f["kernel_ms"] * 1e-3) / 1e9) <= 1e-6 * f["achieved"]
         # the committed counter figures for this workload: at least the algorithmic bytes, not absurdly more
         assert isinstance(f["traffic"], int) and f["algorithmic_bytes"] <= f["traffic"] < 5 * f["algorithmic_bytes"]
+        # (it says where the figure comes from and whether it was measured with the kernel sources of this tree)
+        assert f["traffic_from"].startswith("profiles/") and isinstance(f["traffic_measured_with_these_kernel_sources"], bool)
     assert r["roofline"] == r["roofline_backward"]   # the backward is the longer of the two passes
     assert r["roofline_forward"]["algorithmic_bytes"] == 3584 * queries
     assert r["roofline_backward"]["algorithmic_bytes"] == 6144 * queries
